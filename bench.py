@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the BitStack compressed-linear forward on one MI355X.
+
+Workload ("decode GEMV sweep", the second configuration of the baseline):
+Llama-3.1-8B linear shapes (out x in) 4096x4096, 1024x4096, 14336x4096,
+4096x14336; blocks loaded I in {1, 2, 4, 8, 16}; rank 16; fp16; seeded
+synthetic signs / factors / activations.  One STEP is one pass over all 20
+(shape, I) layers at one token (T = 1) through the library's fused forward
+(C ABI bs_forward), each layer with its own buffers (586 MB per pass, more
+than the 256 MB Infinity Cache, so every pass streams from HBM).
+
+The headline value is the whole-pass throughput in algorithmic GB/s:
+sum over layers of I * (M*N/8 + 2*k*(M+N)) + 2*T*(N+M) bytes, divided by the
+wall time of the timed region (inputs resident in HBM, launches back to back,
+synchronised on both sides).
+
+Extra objects on the same JSON line:
+  roofline      the packed-sign GEMV kernel pair (contraction + partial-sum
+                reduce) against the 8 TB/s HBM peak: algorithmic bytes per
+                forward / HIP-event time per forward, averaged over the timed
+                region (events recorded on the stream the kernels run on).
+  cpu_baseline  the reference's CPU path (level 0) restated in torch-CPU ops,
+                timed on this host on one pass of the same sweep.
+  t4, prefill   the same sweep at 4 tokens, and the prefill configuration
+                (I = 8, T in {16, 128, 512, 2048}) as useful TFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
+BLOCKS = [1, 2, 4, 8, 16]
+PREFILL_T = [16, 128, 512, 2048]
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
+    ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
+    return ap.parse_args()
+
+
+class Layer:
+    def __init__(self, M, N, I, T, seed, dev):
+        import torch
+        from bitstack_amd.utils.synthetic import synthetic_layer, algorithmic_bytes
+        self.M, self.N, self.I, self.T = M, N, I, T
+        self.q, self.u, self.vt, self.x = synthetic_layer(M, N, I, T, seed=seed, device=dev)
+        self.y = torch.empty((T, M), dtype=torch.float16, device=dev)
+        self.bytes = algorithmic_bytes(I, M, N, T)
+
+
+def make_forward(L, lib, ws, stream):
+    """Bind one bs_forward call (C ABI, ctypes) with all arguments resolved."""
+    from bitstack_amd import _lib
+    args = (_lib.ptr(L.q), _lib.ptr(L.u), _lib.ptr(L.vt), _lib.ptr(L.x), None, _lib.ptr(L.y),
+            L.I, L.M, L.N, 16, L.T, _lib.ptr(ws), ws.numel(), stream)
+
+    def run():
+        st = lib.bs_forward(*args)
+        if st != 0:
+            raise RuntimeError(f"bs_forward status {st}: {_lib.error_string(st)}")
+    return run
+
+
+def cpu_baseline(layers_cpu):
+    """One pass of the T=1 sweep through the level-0 restatement on the host."""
+    import torch
+    from oracle import torch_l0
+    threads = os.cpu_count() or 1
+    # the GPU box exposes 16 cores to this job whatever cpu_count() says
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    torch.set_num_threads(threads)
+    tot_b, tot_t = 0, 0.0
+    torch_l0.forward_l0(*layers_cpu[0][:4])          # warm-up
+    for (q, u, vt, x, nbytes) in layers_cpu:
+        t = time.perf_counter()
+        torch_l0.forward_l0(q, u, vt, x)
+        tot_t += time.perf_counter() - t
+        tot_b += nbytes
+    return {"value": round(tot_b / tot_t / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"one pass of the T=1 sweep ({len(layers_cpu)} layers, {tot_b / 1e6:.0f} MB algorithmic, "
+                      f"{tot_t:.1f} s) through the level-0 torch-CPU restatement",
+            "seconds": round(tot_t, 2)}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py: this build measures one GPU; --gpus {a.gpus} is not supported "
+              "(every box in this run has a single MI355X)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from bitstack_amd import _lib
+    from bitstack_amd.utils.synthetic import synthetic_layer, algorithmic_bytes
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.lib()
+    stream = _lib.stream_ptr(dev)
+
+    def build_sweep(T, shapes=SHAPES, blocks=BLOCKS):
+        out, seed = [], 0
+        for (M, N) in shapes:
+            for I in blocks:
+                out.append(Layer(M, N, I, T, seed, dev))
+                seed += 1
+        return out
+
+    def workspace_for(layers):
+        need = max(int(lib.bs_workspace_bytes(L.I, L.M, L.N, 16, L.T)) for L in layers)
+        return torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+
+    def time_sweep(layers, steps, warmup, per_layer_events):
+        ws = workspace_for(layers)
+        fns = [make_forward(L, lib, ws, stream) for L in layers]
+        for _ in range(warmup):
+            for f in fns:
+                f()
+        torch.cuda.synchronize()
+        ev = None
+        if per_layer_events:
+            ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                   for _ in fns] for _ in range(steps)]
+        t0 = time.perf_counter()
+        for s in range(steps):
+            for j, f in enumerate(fns):
+                if ev:
+                    ev[s][j][0].record()
+                f()
+                if ev:
+                    ev[s][j][1].record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        per_layer = None
+        if ev:
+            per_layer = [sum(ev[s][j][0].elapsed_time(ev[s][j][1]) for s in range(steps)) / steps
+                         for j in range(len(fns))]          # ms per forward
+        return wall, per_layer
+
+    # ---------------------------------------------------------------- headline: T = 1 sweep
+    layers = build_sweep(1)
+    pass_bytes = sum(L.bytes for L in layers)
+    # (a) whole-job wall clock, no events in the stream
+    wall, _ = time_sweep(layers, a.steps, a.warmup, per_layer_events=False)
+    ms_per_step = wall / a.steps * 1e3
+    value = pass_bytes * a.steps / wall / 1e9
+    # (b) kernel time per forward from HIP events on the launch stream
+    _, per_layer = time_sweep(layers, a.steps, 1, per_layer_events=True)
+    ev_total_ms = sum(per_layer)
+    achieved = pass_bytes / (ev_total_ms * 1e-3) / 1e9
+    detail = [{"M": L.M, "N": L.N, "I": L.I, "T": L.T, "bytes": L.bytes, "us": round(ms * 1e3, 2),
+               "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(layers, per_layer)]
+    best = max(detail, key=lambda d: d["GBps"])
+
+    out = {
+        "metric": "packed-sign GEMV HBM GB/s (decode sweep, Llama-3.1-8B linear shapes, T=1)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "decode GEMV sweep: (out x in) in {4096x4096, 1024x4096, 14336x4096, 4096x14336} "
+                               "x blocks {1,2,4,8,16}, k=16, T=1, one fused forward per layer, distinct buffers per layer",
+                   "layers_per_step": len(layers), "algorithmic_MB_per_step": round(pass_bytes / 1e6, 1)},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv_kernel<T=1> + gemv_reduce_kernel, averaged over the sweep",
+                     "avg_us_per_forward": round(ev_total_ms * 1e3 / len(layers), 2),
+                     "avg_algorithmic_MB_per_forward": round(pass_bytes / len(layers) / 1e6, 3),
+                     "best_layer": best},
+    }
+
+    if not a.no_extras:
+        # ------------------------------------------------------------ T = 4 sweep (MFMA-bound side)
+        l4 = build_sweep(4)
+        _, per4 = time_sweep(l4, max(3, a.steps // 2), 1, per_layer_events=True)
+        b4 = sum(L.bytes for L in l4)
+        flops4 = sum(2.0 * 16 * L.I * L.M * L.N * L.T for L in l4)
+        t4 = sum(per4) * 1e-3
+        out["t4"] = {"GBps": round(b4 / t4 / 1e9, 1), "mfma_tflops_issued": round(flops4 / t4 / 1e12, 1),
+                     "frac_of_f16_mfma_peak": round(flops4 / t4 / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+        detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 4, "bytes": L.bytes, "us": round(ms * 1e3, 2),
+                    "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l4, per4)]
+        del l4
+        # ------------------------------------------------------------ prefill (useful flops)
+        pre = {}
+        for T in PREFILL_T:
+            lp = build_sweep(T, blocks=[8])
+            _, perp = time_sweep(lp, 3, 1, per_layer_events=True)
+            useful = sum(2.0 * L.M * L.N * L.T + 2.0 * 16 * L.I * L.M * L.N for L in lp)
+            tp = sum(perp) * 1e-3
+            pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
+                            "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+            detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
+                        "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
+                       for L, ms in zip(lp, perp)]
+            del lp
+        out["prefill"] = pre
+
+    if not a.no_cpu_baseline:
+        cpu_layers = []
+        seed = 0
+        for (M, N) in SHAPES:
+            for I in BLOCKS:
+                q, u, vt, x = synthetic_layer(M, N, I, 1, seed=seed)
+                cpu_layers.append((q, u, vt, x, algorithmic_bytes(I, M, N, 1)))
+                seed += 1
+        out["cpu_baseline"] = cpu_baseline(cpu_layers)
+    else:
+        out["cpu_baseline"] = None
+
+    if a.detail:
+        os.makedirs(os.path.dirname(os.path.abspath(a.detail)), exist_ok=True)
+        with open(a.detail, "w") as f:
+            json.dump(detail, f, indent=1)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,103 @@
+"""ctypes binding of libbitstack_hip.so (the C ABI in include/bitstack_hip.h).
+
+There is no CPU fallback: if the shared library is missing, or a tensor is not
+on a HIP device, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+import threading
+
+import torch
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libbitstack_hip.so")
+
+# name -> (restype, argtypes); mirrors include/bitstack_hip.h one to one
+_P, _I, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+SIGNATURES = {
+    "bs_version": (_I, []),
+    "bs_error_string": (ctypes.c_char_p, [_I]),
+    "bs_pack_sign": (_I, [_P, _P, _L, _P]),
+    "bs_unpack_sign": (_I, [_P, _P, _L, _P]),
+    "bs_reconstruct_w_from_sign": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "bs_reconstruct_w": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "bs_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
+    "bs_forward": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _L, _P]),
+    "bs_linear_f16": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+def build(force: bool = True) -> str:
+    """Compile the HIP sources for gfx950 (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", _CSRC, "-j8"] + (["-B"] if force else [])
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        f"{LIB_PATH} is missing: build it with `make -C {_CSRC}` "
+                        "(or __graft_entry__.build()); there is no fallback path")
+                L = ctypes.CDLL(LIB_PATH)
+                for name, (res, args) in SIGNATURES.items():
+                    fn = getattr(L, name)
+                    fn.restype, fn.argtypes = res, args
+                _lib = L
+    return _lib
+
+
+def error_string(status: int) -> str:
+    return lib().bs_error_string(int(status)).decode()
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise RuntimeError(f"{what} failed with status {status}: {error_string(status)}")
+
+
+def require_gpu(*tensors) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("bitstack_amd HIP kernels need tensors on a HIP device; "
+                               f"got a tensor on {t.device} (fused_level 0 is the torch-only path)")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def stream_ptr(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+_workspaces: dict = {}
+
+
+def workspace(dev, nbytes: int):
+    """Per-(device, stream) scratch tensor, grown on demand.  Kernels on one
+    stream are ordered, so reusing it across calls on that stream is safe."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[key] = buf
+    return buf

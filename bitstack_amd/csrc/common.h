@@ -1,0 +1,44 @@
+// Shared host-side helpers for the gfx950 BitStack kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bitstack_hip.h"
+
+#define BS_VERSION_NUMBER 100  // 0.1.0
+
+// Turn a failed HIP call into the documented negative status.
+#define BS_HIP_TRY(expr)                                          \
+    do {                                                          \
+        hipError_t bs_e_ = (expr);                                \
+        if (bs_e_ != hipSuccess) return BS_ERR_HIP_BASE - (int)bs_e_; \
+    } while (0)
+
+// A kernel launch reports configuration errors through hipGetLastError.
+#define BS_LAUNCH_CHECK() BS_HIP_TRY(hipGetLastError())
+
+static inline bool bs_aligned(const void *p, uintptr_t a) {
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+static inline int64_t bs_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+// Internal launchers (one per translation unit), all return a status.
+int bs_launch_reconstruct_packed(const uint8_t *packed, const half_t *u, const half_t *vt,
+                                 half_t *w, int I, int M, int N, int K, hipStream_t s);
+int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, half_t *y,
+                         int T, int M, int N, hipStream_t s);
+int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
+                   const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
+                   void *workspace, int64_t workspace_bytes, hipStream_t s);
+int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T);

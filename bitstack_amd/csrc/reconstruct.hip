@@ -1,0 +1,185 @@
+// Weight reconstruction for gfx950:
+//   w[m, n] = fp16( sum_i s_i[m, n] * sum_r u_i[m, r] * vt_i[r, n] )
+// fp32 everywhere until the single final rounding.
+//
+// Tiled kernel: a workgroup owns 64 rows x 128 columns and walks the blocks.
+// Per block the rank-k product of a 16 x 16 patch is one MFMA
+// (v_mfma_f32_16x16x16_f16) computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
+// so that a lane ends up with four consecutive columns of one row - exactly
+// one nibble of that row's packed sign byte.  The sign is moved to bit 31,
+// merged into the constant 1.0f and applied with one FMA.
+//
+// vt is stored rank-major ([K, N]); the MFMA wants the rank index contiguous
+// per lane, so each block's 16 x 128 slice of vt goes through LDS transposed
+// (column stride 18 halves: 4-byte aligned reads, no bank aliasing between
+// the four 8-column pieces a wave writes at once).
+#include "common.h"
+
+namespace {
+
+constexpr int RT_ROWS = 64;    // rows per workgroup (16 per wave)
+constexpr int RT_COLS = 128;   // columns per workgroup
+constexpr int VSTRIDE = 18;    // halves between consecutive columns in LDS
+
+template <bool PACKED>
+__global__ __launch_bounds__(256) void reconstruct_tile_kernel(
+    const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
+    const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
+    int I, int M, int N, int K) {
+    __shared__ half_t vl[2][RT_COLS * VSTRIDE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * RT_COLS;
+    const int m0 = blockIdx.y * RT_ROWS + wave * 16;
+    const int row = min(m0 + lm, M - 1);
+    const int64_t row_bytes = N >> 3;
+    const int64_t block_bytes = (int64_t)M * row_bytes;
+
+    // staging role: rank index fastest across lanes, 16 pieces of 8 columns
+    const int sr = tid & 15, sp = tid >> 4;
+    // shift that brings this lane's first column of an even 16-column patch to bit 31
+    const int sh_even = 24 - 8 * (g >> 1) + 4 * (g & 1);
+
+    float4_t acc[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    for (int i = 0; i < I; i++) {
+        const int buf = i & 1;
+        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (sr < K)
+            v = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
+#pragma unroll
+        for (int e = 0; e < 8; e++) vl[buf][(8 * sp + e) * VSTRIDE + sr] = v[e];
+
+        half4_t b;   // u_i[row, 4g .. 4g+3], zero beyond the rank
+        {
+            const half_t *up = u + ((int64_t)i * M + row) * K;
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[4 * g + j] : (half_t)0;
+        }
+
+        uint4_t sw = {0, 0, 0, 0};
+        if (PACKED) {
+            sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
+            sw = ~sw;   // bit 1 means +1: make it a clear IEEE sign bit
+        }
+        __syncthreads();
+
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const half_t *ap = &vl[buf][(16 * s + lm) * VSTRIDE + 4 * g];
+            half2_t a01 = *reinterpret_cast<const half2_t *>(ap);
+            half2_t a23 = *reinterpret_cast<const half2_t *>(ap + 2);
+            half4_t a = {a01[0], a01[1], a23[0], a23[1]};
+            float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            if (PACKED) {
+                uint32_t t = sw[s >> 1] << (sh_even - 16 * (s & 1));
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
+                    acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                }
+            } else {
+                uint32_t t = *reinterpret_cast<const uint32_t *>(
+                    sign + ((int64_t)i * M + row) * N + n0 + 16 * s + 4 * g);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
+                    acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                }
+            }
+        }
+    }
+
+    if (m0 + lm < M) {
+        half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 4 * g;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            half4_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
+            *reinterpret_cast<half4_t *>(wp + 16 * s) = o;
+        }
+    }
+}
+
+// Any shape (also rows that do not start on a byte boundary): one output per
+// thread, bit addressed through the flat element index.
+template <bool PACKED>
+__global__ __launch_bounds__(256) void reconstruct_generic_kernel(
+    const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
+    const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
+    int I, int M, int N, int K) {
+    const int64_t total = (int64_t)M * N;
+    const int64_t block_bytes = (total + 7) >> 3;
+    int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; e < total; e += stride) {
+        const int m = (int)(e / N), n = (int)(e % N);
+        float acc = 0.f;
+        for (int i = 0; i < I; i++) {
+            float p = 0.f;
+            for (int r = 0; r < K; r++)
+                p = __builtin_fmaf((float)u[((int64_t)i * M + m) * K + r],
+                                   (float)vt[((int64_t)i * K + r) * N + n], p);
+            float s;
+            if (PACKED)
+                s = ((packed[i * block_bytes + (e >> 3)] >> (7 - (int)(e & 7))) & 1) ? 1.f : -1.f;
+            else
+                s = (float)sign[(int64_t)i * total + e];
+            acc += s * p;
+        }
+        w[e] = (half_t)acc;
+    }
+}
+
+template <bool PACKED>
+int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *u, const half_t *vt,
+                       half_t *w, int I, int M, int N, int K, hipStream_t s) {
+    const bool tiled = (N % RT_COLS == 0) && bs_aligned(vt, 16) && bs_aligned(w, 8) &&
+                       (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
+    if (tiled) {
+        dim3 grid(N / RT_COLS, (unsigned)bs_cdiv(M, RT_ROWS));
+        reconstruct_tile_kernel<PACKED><<<grid, 256, 0, s>>>(packed, sign, u, vt, w, I, M, N, K);
+    } else {
+        int64_t blocks = bs_cdiv((int64_t)M * N, 256);
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        reconstruct_generic_kernel<PACKED><<<(int)blocks, 256, 0, s>>>(packed, sign, u, vt, w, I, M, N, K);
+    }
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
+int check_dims(int I, int M, int N, int K) {
+    if (I < 0 || M <= 0 || N <= 0) return BS_ERR_SHAPE;
+    if (K < 1 || K > 16) return BS_ERR_RANK;
+    if ((int64_t)M * N > ((int64_t)1 << 40)) return BS_ERR_SHAPE;
+    return BS_OK;
+}
+
+}  // namespace
+
+int bs_launch_reconstruct_packed(const uint8_t *packed, const half_t *u, const half_t *vt,
+                                 half_t *w, int I, int M, int N, int K, hipStream_t s) {
+    return launch_reconstruct<true>(packed, nullptr, u, vt, w, I, M, N, K, s);
+}
+
+extern "C" int bs_reconstruct_w(const uint8_t *packed, const void *u, const void *vt, void *w,
+                                int I, int M, int N, int K, void *stream) {
+    int st = check_dims(I, M, N, K);
+    if (st != BS_OK) return st;
+    if (!w || (I > 0 && (!packed || !u || !vt))) return BS_ERR_NULL;
+    if (!bs_aligned(u, 2) || !bs_aligned(vt, 2) || !bs_aligned(w, 2)) return BS_ERR_ALIGN;
+    return launch_reconstruct<true>(packed, nullptr, (const half_t *)u, (const half_t *)vt,
+                                    (half_t *)w, I, M, N, K, (hipStream_t)stream);
+}
+
+extern "C" int bs_reconstruct_w_from_sign(const int8_t *sign, const void *u, const void *vt, void *w,
+                                          int I, int M, int N, int K, void *stream) {
+    int st = check_dims(I, M, N, K);
+    if (st != BS_OK) return st;
+    if (!w || (I > 0 && (!sign || !u || !vt))) return BS_ERR_NULL;
+    if (!bs_aligned(u, 2) || !bs_aligned(vt, 2) || !bs_aligned(w, 2)) return BS_ERR_ALIGN;
+    return launch_reconstruct<false>(nullptr, sign, (const half_t *)u, (const half_t *)vt,
+                                     (half_t *)w, I, M, N, K, (hipStream_t)stream);
+}

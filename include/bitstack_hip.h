@@ -1,0 +1,119 @@
+/*
+ * bitstack_hip.h - C ABI of the MI355X (gfx950) BitStack compressed-linear
+ * forward path.
+ *
+ * Every entry point takes plain device pointers and sizes, returns an int
+ * status (0 = ok, negative = error, see bs_error_string), never throws, never
+ * aborts and never synchronises the host with the device: work is enqueued on
+ * the HIP stream that is passed in (a hipStream_t cast to void*, NULL = the
+ * default stream).  Tensors are dense and row-major exactly as the reference
+ * module stores them after stack_blocks() (bitstack/modules/
+ * BitStackLinear.py:183-195):
+ *
+ *   packed  uint8 [I, M*N/8]  signs, flat row-major over (M, N), first element
+ *                             of every group of eight in the most significant
+ *                             bit, bit 1 = +1, bit 0 = -1
+ *                             (bitstack/utils/pack_utils.py:5-18)
+ *   u       fp16  [I, M, K]
+ *   vt      fp16  [I, K, N]
+ *   x       fp16  [T, N]      y  fp16 [T, M]      bias fp16 [M] or NULL
+ *
+ * with I = blocks loaded (w_bit), M = out_features, N = in_features,
+ * K = rank of a block (1..16), T = tokens.
+ */
+#ifndef BITSTACK_HIP_H
+#define BITSTACK_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BS_OK                 0
+#define BS_ERR_NULL          -1   /* a required pointer is NULL                      */
+#define BS_ERR_SHAPE         -2   /* non-positive or unsupported dimension           */
+#define BS_ERR_RANK          -3   /* K outside 1..16                                 */
+#define BS_ERR_ALIGN         -4   /* pointer not aligned as documented               */
+#define BS_ERR_WORKSPACE     -5   /* workspace missing or smaller than required      */
+#define BS_ERR_NO_DEVICE     -6   /* no HIP device / wrong architecture              */
+#define BS_ERR_HIP_BASE   -1000   /* -(1000 + hipError_t) for a failed HIP call      */
+
+/* Library version, major * 10000 + minor * 100 + patch. */
+int bs_version(void);
+
+/* Static, human readable text for a status returned by any entry point. */
+const char *bs_error_string(int status);
+
+/*
+ * Pack n_elems signs (+-1, int8) into ceil(n_elems/8) bytes; tail bits are 0.
+ * Replaces pack_sign, bitstack/utils/pack_utils.py:5-18.
+ * Entries other than +-1 are not diagnosed on the device: a positive entry
+ * packs as +1, anything else as -1.
+ */
+int bs_pack_sign(const int8_t *sign, uint8_t *packed, int64_t n_elems, void *stream);
+
+/*
+ * Unpack n_elems signs from ceil(n_elems/8) bytes into int8 +-1.
+ * Replaces unpack_sign / unpack_sign_triton + unpack_sign_kernel,
+ * bitstack/utils/pack_utils.py:20-26, :94-138, :177-204.  Bit exact.
+ */
+int bs_unpack_sign(const uint8_t *packed, int8_t *out, int64_t n_elems, void *stream);
+
+/*
+ * w[M, N] (fp16) = sum_i sign_i o (u_i @ vt_i), fp32 accumulation over K and
+ * over the blocks, one rounding to fp16, from ALREADY UNPACKED int8 signs
+ * [I, M, N].  Replaces reconstruct_w_triton + fused_reconstruct_kernel,
+ * bitstack/utils/inference_utils.py:47-115, :135-156.
+ */
+int bs_reconstruct_w_from_sign(const int8_t *sign, const void *u, const void *vt, void *w,
+                               int I, int M, int N, int K, void *stream);
+
+/*
+ * Same result straight from the packed signs.  Replaces
+ * unpack_and_reconstruct_w_triton (+ _v2) and their kernels,
+ * bitstack/utils/inference_utils.py:291-387, :395-488.  Deterministic (no
+ * atomics).  Any M, N (bits are addressed through the flat element index);
+ * the tiled MFMA kernel runs when N % 128 == 0 and the buffers are 16-byte
+ * aligned, a one-output-per-thread kernel otherwise.
+ */
+int bs_reconstruct_w(const uint8_t *packed, const void *u, const void *vt, void *w,
+                     int I, int M, int N, int K, void *stream);
+
+/*
+ * Bytes of device scratch bs_forward needs for these dimensions (0 is a valid
+ * answer); negative = error status.
+ */
+int64_t bs_workspace_bytes(int I, int M, int N, int K, int T);
+
+/*
+ * y[T, M] = x[T, N] @ (sum_i sign_i o (u_i @ vt_i))^T (+ bias), the whole
+ * forward of the layer from packed signs.  Replaces BitStackLinear.forward at
+ * fused levels 1-5 (bitstack/modules/BitStackLinear.py:116-157) including
+ * reconstruct_and_forward_triton + fused_reconstruct_and_forward_kernel
+ * (bitstack/utils/inference_utils.py:171-284).
+ *
+ * T <= 8 runs the packed-sign GEMV (signs contracted on MFMA against
+ * vt_i o x, scaled by u_i, all blocks in one pass); larger T rebuilds the
+ * weight once into `workspace` and runs a dense MFMA GEMM.  Requires
+ * N % 8 == 0.  `workspace` must hold bs_workspace_bytes(...) bytes, 256-byte
+ * aligned; its contents on entry do not matter and it may be reused by the
+ * next call on the same stream.
+ */
+int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void *x,
+               const void *bias, void *y, int I, int M, int N, int K, int T,
+               void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * y[T, M] = x[T, N] @ w[M, N]^T (+ bias) on MFMA, fp32 accumulation: the
+ * dense contraction bs_forward uses for large T, exposed for levels 2-4 where
+ * the reference calls F.linear on the rebuilt weight
+ * (bitstack/modules/BitStackLinear.py:132,140,148).
+ */
+int bs_linear_f16(const void *x, const void *w, const void *bias, void *y,
+                  int T, int M, int N, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BITSTACK_HIP_H */

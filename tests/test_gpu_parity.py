@@ -1,0 +1,267 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, on a real
+MI355X.  Integer / byte work is compared bit for bit; floating point within
+
+    max|d| / max|y_ref| <= 1e-2   and   mean|d| / mean|y_ref| <= 1e-3
+
+against the fp64 closed form and against the level-0 rounding order (the
+tolerance the task states for fp16 layer outputs)."""
+import numpy as np
+import pytest
+import torch
+
+from bitstack_amd import BitStackLinear, _lib
+from bitstack_amd.utils import inference_utils as IU
+from bitstack_amd.utils import pack_utils as PU
+from bitstack_amd.utils.synthetic import synthetic_layer
+from oracle import bitstack_oracle as O
+from oracle import c_oracle as C
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, MEAN_REL = 1e-2, 1e-3
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def rel_errors(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    d = np.abs(got - ref)
+    return d.max() / max(np.abs(ref).max(), 1e-30), d.mean() / max(np.abs(ref).mean(), 1e-30)
+
+
+def assert_close(got, ref, what, max_rel=MAX_REL, mean_rel=MEAN_REL):
+    mx, mn = rel_errors(got, ref)
+    print(f"{what}: max_rel={mx:.3e} mean_rel={mn:.3e}", flush=True)
+    assert mx <= max_rel and mn <= mean_rel, f"{what}: max_rel={mx:.3e} mean_rel={mn:.3e}"
+
+
+def test_library_is_the_hip_build():
+    assert _lib.lib().bs_version() >= 100
+    assert torch.cuda.get_device_properties(0).gcnArchName.startswith("gfx950")
+
+
+# ------------------------------------------------------------------ integers
+@pytest.mark.parametrize("n", [8, 32, 33, 1000, 4096, 64 * 72, 1 << 20, (1 << 20) + 13, 4096 * 4096])
+def test_unpack_bit_exact(n):
+    print(f"unpack n={n}", flush=True)
+    rng = np.random.default_rng(n & 0xFFFF)
+    packed = rng.integers(0, 256, size=(n + 7) // 8, dtype=np.uint8)
+    got = PU.unpack_sign_hip(torch.from_numpy(packed).to(dev()), (n,)).cpu().numpy()
+    want = np.unpackbits(packed, bitorder="big")[:n].astype(np.int8) * 2 - 1
+    assert got.dtype == np.int8 and np.array_equal(got, want)
+    if n <= 1 << 20:
+        assert np.array_equal(got, O.unpack_sign(packed, (n,)))
+
+
+def test_unpack_from_unaligned_views():
+    rng = np.random.default_rng(5)
+    base = torch.from_numpy(rng.integers(0, 256, size=5000, dtype=np.uint8)).to(dev())
+    for off in (1, 2, 3, 5):
+        view = base[off:off + 4000]
+        got = PU.unpack_sign_hip(view, (4000 * 8,)).cpu().numpy()
+        assert np.array_equal(got, O.unpack_sign(view.cpu().numpy(), (32000,)))
+
+
+def test_unpack_all_blocks_shape():
+    q, _, _, _ = synthetic_layer(64, 128, 3, 1, device=dev())
+    s = PU.unpack_sign_triton(q.view(-1), torch.Size([3, 64, 128]))
+    assert tuple(s.shape) == (3, 64, 128)
+    for i in range(3):
+        assert np.array_equal(s[i].cpu().numpy(), O.unpack_sign(q[i].cpu().numpy(), (64, 128)))
+
+
+@pytest.mark.parametrize("shape", [(8,), (5, 7), (13,), (64, 72), (1024, 4096)])
+def test_pack_bit_exact_and_round_trip(shape):
+    print(f"pack shape={shape}", flush=True)
+    rng = np.random.default_rng(len(shape) + shape[0])
+    s = (rng.integers(0, 2, size=shape) * 2 - 1).astype(np.int8)
+    st = torch.from_numpy(s).to(dev())
+    p = PU.pack_sign(st)
+    assert np.array_equal(p.cpu().numpy(), np.packbits((s.reshape(-1) > 0), bitorder="big"))
+    assert torch.equal(PU.unpack_sign(p, torch.Size(shape)), st)
+
+
+# --------------------------------------------------------------- reconstruct
+RECON_CASES = [(1, 64, 128, 16), (3, 64, 256, 16), (2, 50, 128, 16), (4, 256, 512, 16),
+               (2, 64, 128, 7), (1, 64, 128, 1), (2, 40, 72, 16), (3, 33, 100, 5),
+               (8, 1024, 4096, 16)]
+
+
+@pytest.mark.parametrize("I,M,N,K", RECON_CASES)
+def test_reconstruct_w_matches_oracle(I, M, N, K):
+    print(f"reconstruct I={I} M={M} N={N} K={K}", flush=True)
+    q, u, vt, _ = synthetic_layer(M, N, I, 1, k=K, seed=I + M, signed_factors=True)
+    u, vt = (u * 20).half(), (vt * 20).half()
+    want = C.reconstruct_w(q.numpy(), u.numpy(), vt.numpy())
+    qd, ud, vd = q.to(dev()), u.to(dev()), vt.to(dev())
+    got = IU.unpack_and_reconstruct_w_hip(qd, ud, vd).cpu().numpy()
+    assert got.dtype == np.float16 and got.shape == (M, N)
+    # both are one fp16 rounding of an fp32 sum; only the summation order differs
+    ulp = np.spacing(np.abs(want)).astype(np.float64)
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert np.all(diff <= ulp), f"max diff {diff.max()} vs ulp"
+    assert np.mean(diff > 0) < 2e-2
+    assert diff.max() <= 1e-2          # the reference's own self-check bound (atol=1e-2)
+    # the int8-sign entry point gives the identical weight
+    sign = PU.unpack_sign_hip(qd.view(-1), torch.Size([I, M, N]))
+    got2 = IU.reconstruct_w_hip(sign, ud, vd).cpu().numpy()
+    assert np.array_equal(got2.view(np.uint16), got.view(np.uint16))
+
+
+def test_reconstruct_zero_blocks_is_zero():
+    q, u, vt, _ = synthetic_layer(64, 128, 2, 1, device=dev())
+    w = IU.unpack_and_reconstruct_w_hip(q[:0], u[:0], vt[:0])
+    assert float(w.abs().max()) == 0.0
+
+
+# ------------------------------------------------------------------- forward
+def oracle_refs(q, u, vt, x, bias=None):
+    qn, un, vn, xn = q.numpy(), u.numpy(), vt.numpy(), x.numpy()
+    bn = None if bias is None else bias.numpy()
+    return C.forward_f64(qn, un, vn, xn, bn), C.forward_l0(qn, un, vn, xn, bn)
+
+
+GEMV_CASES = [(1, 64, 512, 1), (2, 256, 512, 1), (4, 1024, 1024, 1), (3, 200, 1024, 2),
+              (4, 4096, 4096, 1), (2, 1024, 4096, 4), (8, 4096, 4096, 4), (1, 1024, 4096, 1),
+              (2, 14336, 4096, 1), (2, 4096, 14336, 1), (3, 512, 2048, 3), (2, 512, 1024, 5),
+              (2, 300, 1536, 6), (2, 256, 512, 7), (2, 512, 1024, 8), (16, 1024, 4096, 1)]
+
+
+@pytest.mark.parametrize("I,M,N,T", GEMV_CASES)
+def test_forward_decode_matches_oracle(I, M, N, T):
+    print(f"forward decode I={I} M={M} N={N} T={T}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=I * 7 + T)
+    exact, l0 = oracle_refs(q, u, vt, x)
+    y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())).cpu().numpy()
+    assert y.dtype == np.float16 and y.shape == (T, M)
+    assert_close(y, exact, "vs fp64")
+    assert_close(y, l0, "vs level-0 order")
+
+
+@pytest.mark.parametrize("I,M,N,T,K", [(2, 128, 512, 1, 16), (3, 256, 1024, 2, 5), (2, 64, 512, 1, 1)])
+def test_forward_decode_signed_factors_bias_and_small_rank(I, M, N, T, K):
+    print(f"forward signed I={I} M={M} N={N} T={T} K={K}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=11, signed_factors=True)
+    bias = (torch.randn(M, generator=torch.Generator().manual_seed(1)) * 0.01).half()
+    exact, l0 = oracle_refs(q, u, vt, x, bias)
+    y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev()), bias.to(dev()))
+    assert_close(y.cpu().numpy(), exact, "vs fp64")
+    assert_close(y.cpu().numpy(), l0, "vs level-0 order")
+
+
+@pytest.mark.parametrize("I,M,N,T", [(2, 40, 72, 1), (3, 33, 200, 3), (2, 64, 520, 9), (1, 16, 8, 1)])
+def test_forward_odd_shapes_take_the_rebuild_path(I, M, N, T):
+    print(f"forward odd I={I} M={M} N={N} T={T}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=2)
+    exact, l0 = oracle_refs(q, u, vt, x)
+    y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())).cpu().numpy()
+    assert_close(y, exact, "vs fp64")
+    assert_close(y, l0, "vs level-0 order")
+
+
+PREFILL_CASES = [(2, 256, 512, 16), (8, 1024, 4096, 16), (4, 1024, 1024, 128), (2, 300, 1024, 100),
+                 (8, 4096, 4096, 128), (2, 512, 1024, 512)]
+
+
+@pytest.mark.parametrize("I,M,N,T", PREFILL_CASES)
+def test_forward_prefill_matches_oracle(I, M, N, T):
+    print(f"forward prefill I={I} M={M} N={N} T={T}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=I + T)
+    exact, l0 = oracle_refs(q, u, vt, x)
+    y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())).cpu().numpy()
+    assert y.shape == (T, M)
+    assert_close(y, exact, "vs fp64")
+    assert_close(y, l0, "vs level-0 order")
+
+
+def test_linear_f16_matches_torch_fp32():
+    g = torch.Generator().manual_seed(0)
+    for (T, M, N, b) in [(1, 64, 128, False), (130, 200, 264, True), (256, 256, 512, True), (33, 17, 40, False)]:
+        x = torch.randn(T, N, generator=g).half().to(dev())
+        w = (torch.randn(M, N, generator=g) * 0.05).half().to(dev())
+        bias = torch.randn(M, generator=g).half().to(dev()) if b else None
+        want = x.float() @ w.float().T + (bias.float() if b else 0)
+        got = IU.linear_f16_hip(x, w, bias)
+        assert_close(got.float().cpu().numpy(), want.cpu().numpy(), f"linear {T}x{M}x{N}", 2e-3, 5e-4)
+
+
+# ------------------------------------------------- properties at full size
+def test_full_size_properties_largest_decode_shape():
+    """14336 x 4096 with 16 blocks: too big for the CPU oracle in seconds, so
+    check what must hold whatever the values are."""
+    I, M, N = 16, 14336, 4096
+    q, u, vt, x = synthetic_layer(M, N, I, 1, seed=9, device=dev())
+    f = IU.bitstack_forward_hip
+    y = f(q, u, vt, x).float()
+    # determinism
+    assert torch.equal(f(q, u, vt, x).float(), y)
+    # scaling x by 2 is exact in fp16 and must scale y by exactly 2
+    assert torch.equal(f(q, u, vt, x * 2).float(), 2 * y)
+    # block additivity: the stack equals the sum of its halves (fp16 output rounding only)
+    parts = f(q[:8], u[:8], vt[:8], x).float() + f(q[8:], u[8:], vt[8:], x).float()
+    assert float((parts - y).abs().max()) <= 2e-3 * float(y.abs().max())
+    # complementing the sign bytes of every block negates the output exactly
+    assert torch.equal(f(~q, u, vt, x).float(), -y)
+    # T = 4 rows are the four T = 1 answers
+    x4 = torch.cat([x, x * 0.5, -x, x * 0.25])
+    y4 = f(q, u, vt, x4).float()
+    assert float((y4[0] - y[0]).abs().max()) <= 1e-3 * float(y.abs().max())
+    assert float((y4[2] + y[0]).abs().max()) <= 1e-3 * float(y.abs().max())
+    # spot rows against the fp64 closed form
+    rows = [0, 1, 4095, 7777, 14335]
+    exact = O.forward_exact(np.stack([qq.cpu().numpy().reshape(M, N // 8)[rows].reshape(-1) for qq in q]),
+                            u[:, rows].cpu().numpy(), vt.cpu().numpy(), x.cpu().numpy())
+    assert_close(y[:, rows].cpu().numpy(), exact, "spot rows vs fp64", 1e-2, 2e-3)
+
+
+# ------------------------------------------------------------ module levels
+def build_module(M, N, I, bias, seed):
+    q, u, vt, x = synthetic_layer(M, N, I, 3, seed=seed, signed_factors=True)
+    mod = BitStackLinear(I, N, M, 16, bias, False, "cpu")
+    for i in range(I):
+        getattr(mod, f"qweight_{i}").copy_(q[i])
+        getattr(mod, f"u_{i}").copy_(u[i] * 10)
+        getattr(mod, f"vt_{i}").copy_(vt[i] * 10)
+    if bias:
+        mod.bias.copy_((torch.randn(M, generator=torch.Generator().manual_seed(seed)) * 0.01).half())
+    return mod, x
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_module_levels_agree_with_level0(bias):
+    M, N, I = 256, 1024, 4
+    mod, x = build_module(M, N, I, bias, 21)
+    y0_cpu = mod(x)                                     # level 0 on the CPU
+    mod = mod.to(dev())
+    xd = x.to(dev())
+    y0 = mod(xd)                                        # level 0 on the GPU (torch ops)
+    assert_close(y0.cpu().numpy(), y0_cpu.numpy(), "level0 gpu vs cpu", 2e-3, 5e-4)
+    mod.stack_blocks()
+    for level in (1, 2, 3, 4, 5):
+        mod.fused_level = level
+        y = mod(xd)
+        assert y.dtype == torch.float16 and tuple(y.shape) == (3, M)
+        assert_close(y.cpu().numpy(), y0_cpu.numpy(), f"level {level} vs level 0")
+        y3 = mod(xd.view(1, 3, N))
+        assert tuple(y3.shape) == (1, 3, M) and torch.equal(y3.view(3, M), y)
+    # any-size: fewer blocks through the same stacked buffers
+    mod.fused_level = 5
+    mod.set_bit(2)
+    q2 = torch.stack([mod.qweight[i] for i in range(2)]).cpu()
+    exact = C.forward_f64(q2.numpy(), mod.u[:2].cpu().numpy(), mod.vt[:2].cpu().numpy(), x.numpy(),
+                          None if not bias else mod.bias.cpu().numpy())
+    assert_close(mod(xd).cpu().numpy(), exact, "w_bit=2 vs fp64")
+    mod.set_bit(9)
+    with pytest.raises(RuntimeError, match="exceeds"):
+        mod(xd)
+
+
+def test_non_contiguous_input_is_handled():
+    q, u, vt, x = synthetic_layer(128, 512, 2, 4, seed=4, device=dev())
+    wide = torch.randn(4, 1024, device=dev()).half()
+    wide[:, ::2] = x
+    y = IU.bitstack_forward_hip(q, u, vt, wide[:, ::2])
+    assert torch.equal(y, IU.bitstack_forward_hip(q, u, vt, x))

@@ -1,0 +1,85 @@
+"""CPU-side checks of the shared library: it loads, exports every symbol the
+header declares, and rejects bad arguments with the documented status before
+touching a device (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from bitstack_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bitstack_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bs_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build(force=False)
+    return _lib.lib()
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(_lib.SIGNATURES)
+
+
+def test_every_declared_symbol_is_exported(L):
+    for name in declared_functions():
+        assert hasattr(L, name), name
+
+
+def test_version_and_error_strings(L):
+    assert L.bs_version() >= 100
+    assert _lib.error_string(0) == "ok"
+    for code in (-1, -2, -3, -4, -5, -6):
+        assert _lib.error_string(code) not in ("ok", "unknown status")
+    assert _lib.error_string(-999) == "unknown status"
+
+
+def test_argument_validation_returns_status_not_crash(L):
+    nul = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(256)       # non-null, never dereferenced on these paths
+    odd = ctypes.c_void_p(257)
+    # unpack / pack
+    assert L.bs_unpack_sign(nul, one, 8, nul) == -1
+    assert L.bs_unpack_sign(one, one, -1, nul) == -2
+    assert L.bs_unpack_sign(nul, nul, 0, nul) == 0
+    assert L.bs_pack_sign(one, nul, 8, nul) == -1
+    # reconstruct
+    assert L.bs_reconstruct_w(one, one, one, one, 1, 0, 128, 16, nul) == -2
+    assert L.bs_reconstruct_w(one, one, one, one, 1, 64, 128, 17, nul) == -3
+    assert L.bs_reconstruct_w(one, one, one, one, 1, 64, 128, 0, nul) == -3
+    assert L.bs_reconstruct_w(nul, one, one, one, 1, 64, 128, 16, nul) == -1
+    assert L.bs_reconstruct_w(one, odd, one, one, 1, 64, 128, 16, nul) == -4
+    assert L.bs_reconstruct_w_from_sign(one, one, one, nul, 1, 64, 128, 16, nul) == -1
+    # forward
+    assert L.bs_forward(one, one, one, one, nul, one, 1, 64, 100, 16, 1, one, 1 << 30, nul) == -2   # N % 8
+    assert L.bs_forward(one, one, one, one, nul, one, 1, 64, 128, 32, 1, one, 1 << 30, nul) == -3
+    assert L.bs_forward(one, one, one, nul, nul, one, 1, 64, 128, 16, 1, one, 1 << 30, nul) == -1
+    assert L.bs_forward(odd, one, one, one, nul, one, 1, 64, 128, 16, 1, one, 1 << 30, nul) == -4
+    assert L.bs_forward(one, one, one, one, nul, one, 1, 64, 512, 16, 1, nul, 0, nul) == -5
+    assert L.bs_forward(one, one, one, one, nul, one, 1, 64, 512, 16, 1, one, 16, nul) == -5
+    assert L.bs_forward(one, one, one, one, nul, one, 1, 64, 512, 16, 0, nul, 0, nul) == 0        # T == 0
+    # linear
+    assert L.bs_linear_f16(nul, one, nul, one, 4, 64, 128, nul) == -1
+    assert L.bs_linear_f16(one, one, nul, one, 4, 0, 128, nul) == -2
+
+
+def test_workspace_bytes(L):
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 0) == 0
+    assert L.bs_workspace_bytes(8, 4096, 4100, 16, 1) == -2
+    assert L.bs_workspace_bytes(8, 4096, 4096, 20, 1) == -3
+    # prefill and odd shapes rebuild the fp16 weight
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2
+    assert L.bs_workspace_bytes(2, 64, 72, 16, 1) == ((64 * 72 * 2 + 255) // 256) * 256
+    # decode keeps fp32 partial row sums: a multiple of T * M * 4, far below the weight
+    for T in (1, 4, 8):
+        b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
+        assert b > 0 and b % (T * 4096 * 4) == 0 and b < 4096 * 4096 * 2
