@@ -24,11 +24,9 @@ LLAMA8B_SHAPES = {
 
 
 def synthetic_layer(M, N, I, T, k=16, seed=0, device="cpu", signed_factors=False):
-    """Returns (qweight uint8[I, M*N/8], u f16[I,M,k], vt f16[I,k,N], x f16[T,N])."""
-    if (M * N) % 8:
-        raise ValueError("M * N must be a multiple of 8")
+    """Returns (qweight uint8[I, ceil(M*N/8)], u f16[I,M,k], vt f16[I,k,N], x f16[T,N])."""
     g = torch.Generator().manual_seed(seed)
-    q = torch.randint(0, 256, (I, M * N // 8), dtype=torch.uint8, generator=g)
+    q = torch.randint(0, 256, (I, (M * N + 7) // 8), dtype=torch.uint8, generator=g)
     scale = (0.01 / torch.arange(1, I + 1, dtype=torch.float32)).view(I, 1, 1)
     u = torch.randn(I, M, k, generator=g)
     vt = torch.randn(I, k, N, generator=g)

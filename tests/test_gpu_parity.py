@@ -106,7 +106,8 @@ def test_reconstruct_w_matches_oracle(I, M, N, K):
     assert np.mean(diff > 0) < 2e-2
     assert diff.max() <= 1e-2          # the reference's own self-check bound (atol=1e-2)
     # the int8-sign entry point gives the identical weight
-    sign = PU.unpack_sign_hip(qd.view(-1), torch.Size([I, M, N]))
+    # (unpacked block by block: a block whose M * N is not a multiple of 8 ends in padding bits)
+    sign = torch.stack([PU.unpack_sign_hip(qd[i], torch.Size([M, N])) for i in range(I)])
     got2 = IU.reconstruct_w_hip(sign, ud, vd).cpu().numpy()
     assert np.array_equal(got2.view(np.uint16), got.view(np.uint16))
 
@@ -198,8 +199,9 @@ def test_full_size_properties_largest_decode_shape():
     y = f(q, u, vt, x).float()
     # determinism
     assert torch.equal(f(q, u, vt, x).float(), y)
-    # scaling x by 2 is exact in fp16 and must scale y by exactly 2
-    assert torch.equal(f(q, u, vt, x * 2).float(), 2 * y)
+    # linearity in x (vt * x is rounded to fp16, so products that fall below the
+    # fp16 normal range do not double exactly: compare within the output rounding)
+    assert float((f(q, u, vt, x * 2).float() - 2 * y).abs().max()) <= 2e-3 * float(y.abs().max())
     # block additivity: the stack equals the sum of its halves (fp16 output rounding only)
     parts = f(q[:8], u[:8], vt[:8], x).float() + f(q[8:], u[8:], vt[8:], x).float()
     assert float((parts - y).abs().max()) <= 2e-3 * float(y.abs().max())
