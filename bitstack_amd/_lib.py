@@ -13,7 +13,8 @@ import threading
 import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(_CSRC, "libbitstack_hip.so")
+# BITSTACK_AMD_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("BITSTACK_AMD_LIB") or os.path.join(_CSRC, "libbitstack_hip.so")
 
 # name -> (restype, argtypes); mirrors include/bitstack_hip.h one to one
 _P, _I, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64

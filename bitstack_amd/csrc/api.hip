@@ -43,7 +43,7 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     if (st != BS_OK) return st;
     if (T == 0) return BS_OK;
     if (!x || !y || (I > 0 && (!packed || !u || !vt))) return BS_ERR_NULL;
-    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 2) ||
+    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 8) ||
         !bs_aligned(y, 2) || !bs_aligned(bias, 2))
         return BS_ERR_ALIGN;
     const int64_t need = bs_workspace_bytes(I, M, N, K, T);

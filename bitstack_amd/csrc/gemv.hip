@@ -2,200 +2,464 @@
 //
 //   y[t, m] = sum_i sum_r u_i[m, r] * ( sum_n s_i[m, n] * vt_i[r, n] * x[t, n] )
 //
-// The inner sum is a matrix product  Z_i,t (16 x N)  x  S_i^T (N x rows)  with
-// Z_i,t[r, n] = vt_i[r, n] * x[t, n], so it runs on v_mfma_f32_16x16x32_f16:
-// A = a 16 x 32 patch of Z (fp16), B = 32 signs of 16 rows as fp16 +-1,
-// D[r, m] accumulated in fp32 over the whole slice of n a workgroup owns.  A
-// lane then holds four ranks of ONE row, multiplies them by u_i[m, 4g..4g+3],
-// and two cross-lane adds finish the row.
+// The inner sum is a matrix product  Z (16 ranks x N)  x  S^T (N x rows)  with
+// Z[r, n] = vt_i[r, n] * x[t, n], so it runs on v_mfma_f32_16x16x32_f16:
+// A = a 16 x 32 patch of Z (fp16), B = 32 signs of 16 rows, D[r, m] in fp32.
+// A lane ends up with four ranks of ONE row, multiplies them by
+// u_i[m, 4g..4g+3], and two cross-lane adds finish the row.
 //
-// Work split: workgroup = (row tile of 64*R rows, block i, group of 512-column
-// chunks).  The four waves take 16*R rows each and share Z through LDS; every
-// lane reads its 16 bytes of signs (128 columns of one row) with one 128-bit
-// load per chunk and row tile.  Partial row sums go to a scratch array
-// [I * groups, T, M] (fp32) and a second small kernel adds them in a fixed
-// order, adds the bias and rounds to fp16 - deterministic, no atomics.
+// ---- sign decode without shifts ------------------------------------------
+// Decoding a bit to fp16 +-1 costs a shift and a mask per two signs, which is
+// more VALU time than the MFMA it feeds.  Instead the bit is left WHERE IT IS
+// in its 16-bit half and merged into a constant with one v_and_or_b32:
+//     v = (w & (0x00010001 << j)) | base_j
+// so the fp16 operand is one of two values {a_j, b_j} that depend on the bit
+// position j, chosen such that b_j - a_j = 2 exactly:
+//     j = 15 (sign)        {+1, -1}      mid  0   (Z is stored negated here)
+//     j = 14 (exponent)    {0, 2}        mid  1
+//     j = 9..4 (mantissa)  {4,6} {8,10} {16,18} {32,34} {64,66} {128,130}
+// Then s = v - mid_j, and   sum_n s_n z_n = sum_n v_n z_n - sum_n mid_n z_n.
+// The first sum is what the MFMAs accumulate; the second does not depend on
+// the row and is accumulated by wave 0 with one extra MFMA per step against a
+// constant operand.  All codes are exact in fp16 and every product is exact
+// in fp32, so the only extra error is fp32 accumulation of terms up to 129x
+// larger than z (about 1e-5 relative, far below the fp16 rounding of y).
+// Bit positions 10..13 and 0..3 have no such code (or a badly conditioned
+// one), so the word is used three times: as loaded (positions 15,14,9..4),
+// shifted left by 2 (positions 15,14 = original bits 13,12) and by 4
+// (positions 15,14,7..4 = original bits 11,10,3..0): 2 shifts + 16 merges per
+// 32 signs.
 //
-// Sign decode.  A lane's 16 bytes are four little-endian words w0..w3.  MFMA
-// number c (0..15) of a chunk takes bits c and c+16 of each word: after
-// `w << (15 - c)` they sit in the two fp16 sign positions, and one
-// v_and_or_b32 with 0x80008000 / 0x3C003C00 yields the pair (+-1, +-1).  A set
-// bit thus decodes to -1 whereas the storage format says +1, so Z is produced
-// negated.  Which column a given MFMA k-slot sees follows from this bit
-// choice, and Z is laid out in LDS in exactly that order:
-//   slot s = 2p + h of lane group g in MFMA c  <->  column
-//   128 g + 32 p + 16 h + 8 (c / 8) + 7 - c % 8   of the chunk.
+// ---- work split ------------------------------------------------------------
+// The matrix stack is cut into UNITS: (block i, row tile of WAVES*R*16 rows,
+// 512-column chunk), ordered with the chunk fastest.  The grid is persistent:
+// about two workgroups per CU, each owning one contiguous range of units of
+// equal length, so the load is balanced for any shape and each workgroup pays
+// its pipeline fill once.  Per unit every lane reads its 16 bytes of signs
+// (128 columns of one row) with one 128-bit load per row tile, one unit ahead
+// of use; Z for unit u+1 is produced by all threads (vt and x loads issued
+// before the MFMA loop of unit u, finished after it) into the other half of a
+// double-buffered LDS image laid out in MFMA operand order: one barrier per
+// unit.  Accumulators are flushed whenever the range crosses into another
+// (block, row tile): scaled by u, reduced over ranks, written as a partial
+// row sum to scratch [I, KMAX, T, M] (fp32).  A second kernel adds the
+// partials of a row in a fixed order, adds the bias and rounds to fp16:
+// deterministic, no atomics.  Workgroups with neighbouring ranges - which read
+// the same slices of vt - sit on the same XCD (and share its L2).
 #include "common.h"
+
+#include <type_traits>
+#include <utility>
 
 namespace {
 
+// Compile-time loop: the step tables below must fold to immediates.
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 constexpr int CH = 512;   // columns per chunk: 4 lane groups x 16 bytes of signs
 
-// LDS image of Z for one chunk: [t][c (16)][g (4)][r (16)][slot (8)] halves.
-__device__ inline int z_index(int t, int c, int g, int r) { return (((t * 16 + c) * 4 + g) * 16 + r) * 8; }
 
-template <int T, int R>
-__global__ __launch_bounds__(256) void gemv_kernel(
+// step -> bit position used in that step; steps 0-7 read the word as loaded,
+// 8-9 after `<< 2`, 10-15 after `<< 4`.
+__host__ __device__ constexpr int step_pos(int st) {
+    constexpr int P[16] = {15, 14, 9, 8, 7, 6, 5, 4, 15, 14, 15, 14, 7, 6, 5, 4};
+    return P[st];
+}
+// original bit (within its 16-bit half) -> step that consumes it
+__host__ __device__ constexpr int bit_step(int b) {
+    constexpr int S[16] = {15, 14, 13, 12, 7, 6, 5, 4, 3, 2, 11, 10, 9, 8, 1, 0};
+    return S[b];
+}
+__host__ __device__ constexpr uint32_t pos_base(int j) {
+    return j == 15 ? 0x3C003C00u : j == 14 ? 0u : j == 9 ? 0x44004400u : j == 8 ? 0x48004800u
+         : j == 7 ? 0x4C004C00u : j == 6 ? 0x50005000u : j == 5 ? 0x54005400u : 0x58005800u;
+}
+__host__ __device__ constexpr float pos_mid(int j) {
+    return j == 15 ? 0.f : j == 14 ? 1.f : j == 9 ? 5.f : j == 8 ? 9.f : j == 7 ? 17.f
+         : j == 6 ? 33.f : j == 5 ? 65.f : 129.f;
+}
+
+// mid of the position each step reads (0 for the sign position)
+__constant__ float step_mid_table[16] = {0.f, 1.f, 5.f, 9.f, 17.f, 33.f, 65.f, 129.f,
+                                         0.f, 1.f, 0.f, 1.f, 17.f, 33.f, 65.f, 129.f};
+
+// LDS image of Z for one chunk: [t][step (16)][g (4)][r (16)][slot (8)] halves.
+__device__ inline int z_index(int t, int st, int g, int r) { return (((t * 16 + st) * 4 + g) * 16 + r) * 8; }
+
+__device__ inline uint32_t and_or(uint32_t w, uint32_t mask, uint32_t base) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(w), "s"(mask), "v"(base));
+    return d;
+}
+
+__device__ inline uint32_t pin_vgpr(uint32_t c) {
+    uint32_t d;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(d) : "s"(c));   // opaque: stays in one register
+    return d;
+}
+
+struct Bases {
+    uint32_t b15, b9, b8, b7, b6, b5, b4;
+    __device__ inline uint32_t get(int j) const {
+        return j == 15 ? b15 : j == 9 ? b9 : j == 8 ? b8 : j == 7 ? b7 : j == 6 ? b6 : j == 5 ? b5 : b4;
+    }
+};
+
+// One producer item: rank r, lane group pg, word p, byte pair (JB, JB + 2) of
+// the word.  Two 16-byte pieces of vt (8 consecutive columns each) times x
+// give 8 (slot 2p, slot 2p+1) pairs, one per bit of the byte.
+template <int JB>
+__device__ inline void produce_finish(half_t *zt, int pg, int p, int r, half8_t v0, half8_t v1,
+                                      half8_t x0, half8_t x1) {
+    const half8_t z0 = v0 * x0, z1 = v1 * x1;
+    static_for<8>([&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        constexpr int st = bit_step(8 * JB + 7 - e);
+        constexpr bool neg = step_pos(st) == 15;
+        half2_t o = {z0[e], z1[e]};
+        if (neg) o = -o;
+        *reinterpret_cast<half2_t *>(zt + z_index(0, st, pg, r) + 2 * p) = o;
+    });
+}
+
+// Static partition of U units over G workgroups: the first `rem` get q + 1.
+struct Split {
+    int q, rem;
+    __host__ __device__ int start(int w) const { return w * q + (w < rem ? w : rem); }
+    __host__ __device__ int owner(int unit) const {
+        const int big = rem * (q + 1);
+        return unit < big ? unit / (q + 1) : rem + (unit - big) / q;
+    }
+};
+
+template <int T, int WAVES, int R>
+__global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? 2 : 1))) void gemv_kernel(
     const uint8_t *__restrict__ packed, const half_t *__restrict__ u, const half_t *__restrict__ vt,
     const half_t *__restrict__ x, float *__restrict__ part,
-    int I, int M, int N, int K, int row_tiles, int groups, int chunks_per_group, int n_chunks) {
-    extern __shared__ __attribute__((aligned(16))) half_t zl[];   // T * 16 KB
+    int M, int N, int K, int row_tiles, int n_chunks, Split sp, int kmax) {
+    constexpr int RW = WAVES * R * 16;          // rows per workgroup
+    constexpr int COMBOS = 8 / WAVES;           // (jb, pg) producer combos per wave
+    constexpr int ZHALVES = T * 16 * 4 * 16 * 8;   // one Z buffer
+    constexpr int CSTEPS = 16 / WAVES;          // correction steps handled by each wave
+    extern __shared__ __attribute__((aligned(16))) half_t lds[];
+    half_t *zl = lds;                                              // [2][ZHALVES]
+    float *corrl = reinterpret_cast<float *>(lds + 2 * ZHALVES);   // [WAVES][T][16]
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, keep it scalar
     const int lm = lane & 15, g = lane >> 4;
-    const int rt = blockIdx.x % row_tiles;
-    const int task = blockIdx.x / row_tiles;          // = i * groups + cg
-    const int i = task / groups, cg = task % groups;
-    const int c_begin = cg * chunks_per_group;
-    const int c_end = min(c_begin + chunks_per_group, n_chunks);
+
+    // XCD-aware slot -> range: hardware deals workgroups round-robin to 8 XCDs;
+    // give each XCD a contiguous run of ranges.
+    int wg;
+    {
+        const int nb = gridDim.x, xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+        const int base = nb >> 3, rem = nb & 7;
+        wg = xcd * base + min(xcd, rem) + loc;
+    }
+    const int u_begin = sp.start(wg), u_end = sp.start(wg + 1);
+    if (u_begin >= u_end) return;
 
     const int64_t row_bytes = N >> 3;
-    const uint8_t *qi = packed + (int64_t)i * M * row_bytes;
-    const half_t *vti = vt + (int64_t)i * K * N;
+    const int pp = lane & 3, pr = lane >> 2;      // producer role: word, rank
+    const bool r_live = pr < K;
 
-    int rowbase[R];
-    const uint8_t *qrow[R];
+    // Addresses are a wave-uniform base (block i, kept in scalar registers) plus a
+    // 32-bit per-lane byte offset that only changes with the row tile.
+    const uint8_t *qbase;       // packed signs of block i
+    const half_t *vbase;
+    uint32_t qoff[R];           // this lane's row in each row tile of the wave
+    const uint32_t voff = ((uint32_t)(r_live ? pr : 0) * (uint32_t)N + 32u * pp) * 2u;   // producer role
+    auto set_row = [&](int rowid) {
+        const int i = rowid / row_tiles, rt = rowid % row_tiles;
+        qbase = packed + (int64_t)i * M * row_bytes;
+        vbase = vt + (int64_t)i * K * N;
 #pragma unroll
-    for (int jr = 0; jr < R; jr++) {
-        rowbase[jr] = rt * (64 * R) + (wave * R + jr) * 16;
-        qrow[jr] = qi + (int64_t)min(rowbase[jr] + lm, M - 1) * row_bytes + 16 * g;
-    }
+        for (int jr = 0; jr < R; jr++) {
+            const uint32_t row = (uint32_t)min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
+            qoff[jr] = row * (uint32_t)row_bytes + 16u * g;
+        }
+    };
+    auto mid_operand = [&](int k) {   // constant MFMA operand for the correction sums of this wave's steps
+        const half_t m = (half_t)step_mid_table[wave * CSTEPS + k];
+        return (half8_t){m, m, m, m, m, m, m, m};
+    };
+
+    Bases bs;
+    bs.b15 = pin_vgpr(pos_base(15)); bs.b9 = pin_vgpr(pos_base(9)); bs.b8 = pin_vgpr(pos_base(8));
+    bs.b7 = pin_vgpr(pos_base(7));   bs.b6 = pin_vgpr(pos_base(6)); bs.b5 = pin_vgpr(pos_base(5));
+    bs.b4 = pin_vgpr(pos_base(4));
 
     float4_t acc[R][T];
+    float4_t corr[T];
+    auto clear_acc = [&]() {
 #pragma unroll
-    for (int jr = 0; jr < R; jr++)
+        for (int t = 0; t < T; t++) {
+            corr[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int t = 0; t < T; t++) acc[jr][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            for (int jr = 0; jr < R; jr++) acc[jr][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    clear_acc();
 
-    for (int c = c_begin; c < c_end; c++) {
-        const int cb = c * CH;
-        // signs first: their latency hides behind the production of Z
-        uint4_t sw[R];
+    half8_t pv[COMBOS][2];        // vt pieces in flight for the next unit
+    half8_t px[COMBOS][T][2];     // x pieces in flight for the next unit
+    auto produce_issue = [&](int c) {
 #pragma unroll
-        for (int jr = 0; jr < R; jr++) sw[jr] = *reinterpret_cast<const uint4_t *>(qrow[jr] + (cb >> 3));
-
-        if (c != c_begin) __syncthreads();   // everyone is done reading the previous Z
-        for (int item = tid; item < T * 128; item += 256) {
-            const int r = item & 15, pg = (item >> 4) & 3, jb = (item >> 6) & 1, t = item >> 7;
-            half8_t z[8];
+        for (int k = 0; k < COMBOS; k++) {
+            const int combo = wave + k * WAVES, pg = combo & 3, jb = combo >> 2;
+            const int col = c * CH + 128 * pg + 8 * jb;            // wave-uniform
+            const uint8_t *vs = reinterpret_cast<const uint8_t *>(vbase + col) + voff;
+            pv[k][0] = *reinterpret_cast<const half8_t *>(vs);
+            pv[k][1] = *reinterpret_cast<const half8_t *>(vs + 32);
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const int noff = cb + 128 * pg + 32 * (s >> 1) + 16 * (s & 1) + 8 * jb;
-                half8_t xv = *reinterpret_cast<const half8_t *>(x + (int64_t)t * N + noff);
-                half8_t vv = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (r < K) vv = *reinterpret_cast<const half8_t *>(vti + (int64_t)r * N + noff);
-                z[s] = -(vv * xv);
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                half8_t o = {z[0][e], z[1][e], z[2][e], z[3][e], z[4][e], z[5][e], z[6][e], z[7][e]};
-                *reinterpret_cast<half8_t *>(&zl[z_index(t, 8 * jb + 7 - e, pg, r)]) = o;
+            for (int t = 0; t < T; t++) {
+                const uint8_t *xs = reinterpret_cast<const uint8_t *>(x + (int64_t)t * N + col) + 64u * pp;
+                px[k][t][0] = *reinterpret_cast<const half8_t *>(xs);
+                px[k][t][1] = *reinterpret_cast<const half8_t *>(xs + 32);
             }
         }
-        __syncthreads();
-
+    };
+    auto produce_write = [&](int buf) {
+        half_t *zbuf = zl + buf * ZHALVES;
 #pragma unroll
-        for (int cls = 0; cls < 16; cls++) {
+        for (int k = 0; k < COMBOS; k++) {
+            const int combo = wave + k * WAVES, pg = combo & 3, jb = combo >> 2;
+            half8_t v0 = pv[k][0], v1 = pv[k][1];
+            if (!r_live) { v0 = (half8_t){0, 0, 0, 0, 0, 0, 0, 0}; v1 = v0; }
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                half_t *zt = zbuf + z_index(t, 0, 0, 0);
+                if (jb) produce_finish<1>(zt, pg, pp, pr, v0, v1, px[k][t][0], px[k][t][1]);
+                else    produce_finish<0>(zt, pg, pp, pr, v0, v1, px[k][t][0], px[k][t][1]);
+            }
+        }
+    };
+
+    auto consume = [&](uint4_t (&w)[R], int buf) {
+        const half_t *zbuf = zl + buf * ZHALVES;
+        static_for<16>([&](auto stc) {
+            constexpr int st = decltype(stc)::value;
+            if (st == 8 || st == 10) {
+#pragma unroll
+                for (int jr = 0; jr < R; jr++) w[jr] = w[jr] << 2;
+            }
+            constexpr int j = step_pos(st);
+            constexpr uint32_t mask = 0x00010001u << j;
             half8_t zf[T];
 #pragma unroll
-            for (int t = 0; t < T; t++) zf[t] = *reinterpret_cast<const half8_t *>(&zl[z_index(t, cls, g, lm)]);
+            for (int t = 0; t < T; t++) zf[t] = *reinterpret_cast<const half8_t *>(zbuf + z_index(t, st, g, lm));
 #pragma unroll
             for (int jr = 0; jr < R; jr++) {
                 uint4_t sb;
 #pragma unroll
-                for (int p = 0; p < 4; p++) sb[p] = ((sw[jr][p] << (15 - cls)) & 0x80008000u) | 0x3C003C00u;
+                for (int p = 0; p < 4; p++) sb[p] = (j == 14) ? (w[jr][p] & mask) : and_or(w[jr][p], mask, bs.get(j));
                 const half8_t sf = __builtin_bit_cast(half8_t, sb);
 #pragma unroll
                 for (int t = 0; t < T; t++)
                     acc[jr][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zf[t], sf, acc[jr][t], 0, 0, 0);
             }
+        });
+        // row-independent correction: this wave's share of the 16 steps
+#pragma unroll
+        for (int k = 0; k < CSTEPS; k++) {
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                const half8_t zc = *reinterpret_cast<const half8_t *>(zbuf + z_index(t, wave * CSTEPS + k, g, lm));
+                corr[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zc, mid_operand(k), corr[t], 0, 0, 0);
+            }
         }
-    }
+    };
 
-    // D[r, m]: this lane holds ranks 4g..4g+3 of row rowbase + lm
+    auto load_signs = [&](uint4_t (&w)[R], int c) {
 #pragma unroll
-    for (int jr = 0; jr < R; jr++) {
-        const int row = rowbase[jr] + lm;
-        const half_t *up = u + ((int64_t)i * M + min(row, M - 1)) * K + 4 * g;
-        float uf[4];
+        for (int jr = 0; jr < R; jr++) w[jr] = *reinterpret_cast<const uint4_t *>(qbase + c * (CH >> 3) + qoff[jr]);
+    };
+
+    // D[r, m]: the lane holds ranks 4g..4g+3 of row (tile jr, lm).  Subtract the
+    // correction (summed over waves in a fixed order), scale by u, add the four
+    // lane groups, write the partial row sum, start the next row from zero.
+    auto flush = [&](int rowid) {
+        const int i = rowid / row_tiles, rt = rowid % row_tiles;
+        half4_t uc[R];      // u[i, row, 4g .. 4g+3]
 #pragma unroll
-        for (int v = 0; v < 4; v++) uf[v] = (4 * g + v < K) ? (float)up[v] : 0.f;
+        for (int jr = 0; jr < R; jr++) {
+            const int row = min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
+            const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+            if (K == 16) {
+                uc[jr] = *reinterpret_cast<const half4_t *>(up);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; v++) uc[jr][v] = (4 * g + v < K) ? up[v] : (half_t)0;
+            }
+        }
+        if (lm == 0) {
+#pragma unroll
+            for (int t = 0; t < T; t++) *reinterpret_cast<float4_t *>(corrl + (wave * T + t) * 16 + 4 * g) = corr[t];
+        }
+        __syncthreads();
+        const int slot = wg - sp.owner(rowid * n_chunks);
 #pragma unroll
         for (int t = 0; t < T; t++) {
-            float val = acc[jr][t][0] * uf[0] + acc[jr][t][1] * uf[1] + acc[jr][t][2] * uf[2] + acc[jr][t][3] * uf[3];
-            val += __shfl_xor(val, 16, 64);
-            val += __shfl_xor(val, 32, 64);
-            if (g == 0 && row < M) part[((int64_t)task * T + t) * M + row] = val;
+            float4_t cz = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) cz += *reinterpret_cast<const float4_t *>(corrl + (w * T + t) * 16 + 4 * g);
+#pragma unroll
+            for (int jr = 0; jr < R; jr++) {
+                const int row = rt * RW + (wave * R + jr) * 16 + lm;
+                float val = (acc[jr][t][0] - cz[0]) * (float)uc[jr][0] + (acc[jr][t][1] - cz[1]) * (float)uc[jr][1] +
+                            (acc[jr][t][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][t][3] - cz[3]) * (float)uc[jr][3];
+                val += __shfl_xor(val, 16, 64);
+                val += __shfl_xor(val, 32, 64);
+                if (g == 0 && row < M) part[(((int64_t)i * kmax + slot) * T + t) * M + row] = val;
+            }
         }
+        clear_acc();
+    };
+
+    // ---- pipeline fill: first unit's signs and Z -----------------------------
+    int rowid = u_begin / n_chunks, c = u_begin % n_chunks;
+    set_row(rowid);
+    uint4_t cur[R], nxt[R];
+    load_signs(cur, c);
+    produce_issue(c);
+    produce_write(0);
+    __syncthreads();
+
+    // ---- steady state -------------------------------------------------------
+    int buf = 0;
+    for (int unit = u_begin; unit + 1 < u_end; unit++) {
+        const bool crossing = c + 1 == n_chunks;    // the next unit starts another row
+        const int cn = crossing ? 0 : c + 1;
+        if (crossing) set_row(rowid + 1);           // address arithmetic only
+        load_signs(nxt, cn);
+        produce_issue(cn);
+        __builtin_amdgcn_sched_barrier(0);          // keep the prefetch at the top of the unit
+        consume(cur, buf);
+        __builtin_amdgcn_sched_barrier(0);
+        produce_write(buf ^ 1);
+        __syncthreads();
+        if (crossing) {
+            flush(rowid);
+            rowid++;
+        }
+#pragma unroll
+        for (int jr = 0; jr < R; jr++) cur[jr] = nxt[jr];
+        c = cn;
+        buf ^= 1;
     }
+    // ---- drain: last unit, nothing left to prefetch -----------------------------
+    consume(cur, buf);
+    flush(rowid);
 }
 
-// y[t, m] = fp16( sum_k part[k, t, m] + bias[m] ), k ascending.
+// y[t, m] = fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) where k runs over the
+// workgroups whose unit range touched (block i, row tile of m), in ascending
+// order.  One thread per output.
 __global__ __launch_bounds__(256) void gemv_reduce_kernel(const float *__restrict__ part,
                                                           const half_t *__restrict__ bias,
-                                                          half_t *__restrict__ y, int KP, int T, int M) {
+                                                          half_t *__restrict__ y, int I, int T, int M,
+                                                          int rows_per_tile, int row_tiles, int n_chunks,
+                                                          Split sp, int kmax) {
     const int64_t total = (int64_t)T * M;
     const int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (o >= total) return;
+    const int t = (int)(o / M), m = (int)(o % M);
+    const int rt = m / rows_per_tile;
     float acc = 0.f;
-    for (int k = 0; k < KP; k++) acc += part[(int64_t)k * total + o];
-    if (bias) acc += (float)bias[o % M];
+    for (int i = 0; i < I; i++) {
+        const int first = (i * row_tiles + rt) * n_chunks;
+        const int nk = sp.owner(first + n_chunks - 1) - sp.owner(first) + 1;
+        for (int k = 0; k < nk; k++) acc += part[(((int64_t)i * kmax + k) * T + t) * M + m];
+    }
+    if (bias) acc += (float)bias[m];
     y[o] = (half_t)acc;
 }
 
 struct Plan {
-    int R, row_tiles, groups, chunks_per_group, n_chunks;
+    int waves, R, row_tiles, n_chunks, units, grid, kmax;
+    Split sp;
 };
 
-Plan make_plan(int I, int M, int N) {
+Plan make_plan(int I, int M, int N, int T) {
     Plan p;
     p.n_chunks = N / CH;
-    const int64_t want = 768;   // workgroups that keep 256 CUs busy with some slack
-    p.R = 1;
-    for (int r = 4; r >= 1; r >>= 1) {
-        if (bs_cdiv(M, 64 * r) * I * p.n_chunks >= want || r == 1) { p.R = r; break; }
+    // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU
+    const int cand[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
+    int pick = 3;
+    // three or four tokens need more than the 256 registers an 8-wave workgroup can have
+    for (int k = (T > 2 ? 1 : 0); k < 4; k++) {
+        const int rw = cand[k][0] * cand[k][1] * 16;
+        // enough units that every CU gets a few per resident workgroup
+        if (M >= rw && bs_cdiv(M, rw) * I * p.n_chunks >= 2 * 256 * cand[k][2]) { pick = k; break; }
     }
-    p.row_tiles = (int)bs_cdiv(M, 64 * p.R);
-    // merge chunks into groups while enough workgroups remain
-    int cpg = 1;
-    while (cpg * 2 <= p.n_chunks && (int64_t)p.row_tiles * I * bs_cdiv(p.n_chunks, cpg * 2) >= want) cpg *= 2;
-    p.chunks_per_group = cpg;
-    p.groups = (int)bs_cdiv(p.n_chunks, cpg);
+    p.waves = cand[pick][0];
+    p.R = cand[pick][1];
+    p.row_tiles = (int)bs_cdiv(M, p.waves * p.R * 16);
+    p.units = I * p.row_tiles * p.n_chunks;
+    int grid = 256 * (T == 1 ? cand[pick][2] : T == 2 ? 2 : 1);
+    if (grid > p.units / 2) grid = p.units / 2;      // at least two units per workgroup
+    if (grid < 1) grid = 1;
+    p.grid = grid;
+    p.sp.q = p.units / grid;
+    p.sp.rem = p.units % grid;
+    // most workgroups a row of n_chunks units can be spread over
+    int kmax = (int)bs_cdiv(p.n_chunks - 1, p.sp.q) + 1;
+    if (kmax > grid) kmax = grid;
+    p.kmax = kmax;
     return p;
+}
+
+template <int T, int WAVES, int R>
+int launch_one(const Plan &p, const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
+               float *part, int M, int N, int K, hipStream_t s) {
+    const size_t lds = (size_t)2 * T * 16384 + (size_t)WAVES * T * 64;
+    static bool raised = false;      // per instantiation; raising the limit is idempotent
+    if (lds > 64 * 1024 && !raised) {
+        BS_HIP_TRY(hipFuncSetAttribute((const void *)gemv_kernel<T, WAVES, R>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    gemv_kernel<T, WAVES, R><<<p.grid, 64 * WAVES, lds, s>>>(packed, u, vt, x, part, M, N, K, p.row_tiles,
+                                                            p.n_chunks, p.sp, p.kmax);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
 }
 
 template <int T>
 int launch_T(const Plan &p, const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-             float *part, int I, int M, int N, int K, hipStream_t s) {
-    const int grid = p.row_tiles * I * p.groups;
-    const size_t lds = (size_t)T * 16 * 1024;
-#define BS_GEMV_LAUNCH(RR)                                                                        \
-    do {                                                                                          \
-        if (lds > 48 * 1024)                                                                      \
-            BS_HIP_TRY(hipFuncSetAttribute((const void *)gemv_kernel<T, RR>,                       \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
-        gemv_kernel<T, RR><<<grid, 256, lds, s>>>(packed, u, vt, x, part, I, M, N, K, p.row_tiles, \
-                                                  p.groups, p.chunks_per_group, p.n_chunks);      \
-    } while (0)
-    if (p.R == 4) BS_GEMV_LAUNCH(4);
-    else if (p.R == 2) BS_GEMV_LAUNCH(2);
-    else BS_GEMV_LAUNCH(1);
-#undef BS_GEMV_LAUNCH
-    BS_LAUNCH_CHECK();
-    return BS_OK;
+             float *part, int M, int N, int K, hipStream_t s) {
+    if (p.waves == 8) {
+        if constexpr (T <= 2) return launch_one<T, 8, 4>(p, packed, u, vt, x, part, M, N, K, s);
+        else return BS_ERR_SHAPE;     // the planner never pairs 8 waves with more than two tokens
+    }
+    if (p.R == 4) return launch_one<T, 4, 4>(p, packed, u, vt, x, part, M, N, K, s);
+    if (p.R == 2) return launch_one<T, 4, 2>(p, packed, u, vt, x, part, M, N, K, s);
+    return launch_one<T, 4, 1>(p, packed, u, vt, x, part, M, N, K, s);
 }
 
 }  // namespace
 
 static bool gemv_shape_ok(int I, int M, int N, int T) {
-    return I >= 1 && T >= 1 && T <= 8 && N % CH == 0 && M >= 1;
+    // per-block byte offsets are kept in 32 bits inside the kernel
+    return I >= 1 && T >= 1 && T <= 8 && N % CH == 0 && M >= 1 && (int64_t)M * N < ((int64_t)1 << 31);
 }
+
+// Tokens are processed in passes of at most four (LDS holds Z for four tokens).
+static int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
 
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T) {
     (void)K;
     if (!gemv_shape_ok(I, M, N, T)) return 0;
-    Plan p = make_plan(I, M, N);
-    return (int64_t)I * p.groups * T * M * (int64_t)sizeof(float);
+    Plan p = make_plan(I, M, N, pass_tokens(T));
+    return (int64_t)I * p.kmax * pass_tokens(T) * M * (int64_t)sizeof(float);
 }
 
 // Returns BS_ERR_SHAPE when the fast path does not apply (the caller falls
@@ -204,25 +468,28 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
                    const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
                    void *workspace, int64_t workspace_bytes, hipStream_t s) {
     if (!gemv_shape_ok(I, M, N, T)) return BS_ERR_SHAPE;
-    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16)) return BS_ERR_SHAPE;
-    Plan p = make_plan(I, M, N);
-    const int64_t need = (int64_t)I * p.groups * T * M * (int64_t)sizeof(float);
+    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 8)) return BS_ERR_SHAPE;
+    const int64_t need = bs_gemv_workspace_bytes(I, M, N, K, T);
     if (!workspace || workspace_bytes < need) return BS_ERR_WORKSPACE;
     float *part = (float *)workspace;
-    int st;
-    switch (T) {
-        case 1: st = launch_T<1>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 2: st = launch_T<2>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 3: st = launch_T<3>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 4: st = launch_T<4>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 5: st = launch_T<5>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 6: st = launch_T<6>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        case 7: st = launch_T<7>(p, packed, u, vt, x, part, I, M, N, K, s); break;
-        default: st = launch_T<8>(p, packed, u, vt, x, part, I, M, N, K, s); break;
+    const int tp = pass_tokens(T);
+    const Plan p = make_plan(I, M, N, tp);
+    for (int t0 = 0; t0 < T; t0 += tp) {
+        const int tn = (T - t0 < tp) ? T - t0 : tp;
+        const half_t *xp = x + (int64_t)t0 * N;
+        int st;
+        switch (tn) {
+            case 1: st = launch_T<1>(p, packed, u, vt, xp, part, M, N, K, s); break;
+            case 2: st = launch_T<2>(p, packed, u, vt, xp, part, M, N, K, s); break;
+            case 3: st = launch_T<3>(p, packed, u, vt, xp, part, M, N, K, s); break;
+            default: st = launch_T<4>(p, packed, u, vt, xp, part, M, N, K, s); break;
+        }
+        if (st != BS_OK) return st;
+        const int64_t total = (int64_t)tn * M;
+        gemv_reduce_kernel<<<(int)bs_cdiv(total, 256), 256, 0, s>>>(part, bias, y + (int64_t)t0 * M, I, tn, M,
+                                                                   p.waves * p.R * 16, p.row_tiles, p.n_chunks,
+                                                                   p.sp, p.kmax);
+        BS_LAUNCH_CHECK();
     }
-    if (st != BS_OK) return st;
-    const int64_t total = (int64_t)T * M;
-    gemv_reduce_kernel<<<(int)bs_cdiv(total, 256), 256, 0, s>>>(part, bias, y, I * p.groups, T, M);
-    BS_LAUNCH_CHECK();
     return BS_OK;
 }

@@ -205,8 +205,9 @@ def test_full_size_properties_largest_decode_shape():
     # block additivity: the stack equals the sum of its halves (fp16 output rounding only)
     parts = f(q[:8], u[:8], vt[:8], x).float() + f(q[8:], u[8:], vt[8:], x).float()
     assert float((parts - y).abs().max()) <= 2e-3 * float(y.abs().max())
-    # complementing the sign bytes of every block negates the output exactly
-    assert torch.equal(f(~q, u, vt, x).float(), -y)
+    # complementing the sign bytes of every block negates the output (the decode is
+    # not symmetric in the bit value, so only up to fp32 summation order)
+    assert float((f(~q, u, vt, x).float() + y).abs().max()) <= 1e-3 * float(y.abs().max())
     # T = 4 rows are the four T = 1 answers
     x4 = torch.cat([x, x * 0.5, -x, x * 0.25])
     y4 = f(q, u, vt, x4).float()
