@@ -367,36 +367,44 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
 
 // y[t, m] = fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) where k runs over the
 // workgroups whose unit range touched (block i, row tile of m), in ascending
-// order.  64 outputs per workgroup; four threads per output take every fourth
-// block and are combined through LDS in a fixed order.
-__global__ __launch_bounds__(256) void gemv_reduce_kernel(const float *__restrict__ part,
-                                                          const half_t *__restrict__ bias,
-                                                          half_t *__restrict__ y, int I, int T, int M,
-                                                          int rows_per_tile, int row_tiles, int n_chunks,
-                                                          Split sp, int kmax) {
-    __shared__ float red[4][64];
-    const int64_t total = (int64_t)T * M;
-    const int lo = threadIdx.x & 63, ks = threadIdx.x >> 6;
-    const int64_t o = (int64_t)blockIdx.x * 64 + lo;
+// order.  32 outputs of one row tile per workgroup; the number of partials of
+// every block is worked out once (one thread per block) into LDS, eight
+// threads per output take every eighth block (their loads are independent)
+// and are combined through LDS in a fixed order.
+constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;
+
+__global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
+    const float *__restrict__ part, const half_t *__restrict__ bias, half_t *__restrict__ y,
+    int I, int T, int M, int rows_per_tile, int row_tiles, int n_chunks, Split sp, int kmax) {
+    __shared__ int nks[RED_MAXBLOCKS];           // live partials of block i for this row tile
+    __shared__ float red[RED_SL][RED_OUT];
+    const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
+    // outputs are enumerated per token in runs of RED_OUT rows, so a workgroup never straddles tokens
+    const int per_t = (M + RED_OUT - 1) / RED_OUT;
+    const int t = blockIdx.x / per_t, m0 = (blockIdx.x - t * per_t) * RED_OUT, m = m0 + lo;
+    const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
+    for (int i = threadIdx.x; i < I; i += RED_OUT * RED_SL) {
+        const int first = (i * row_tiles + rt) * n_chunks;
+        nks[i] = sp.owner(first + n_chunks - 1) - sp.owner(first) + 1;
+    }
+    __syncthreads();
     float acc = 0.f;
-    int m = 0;
-    if (o < total) {
-        const int t = (int)(o / M);
-        m = (int)(o - (int64_t)t * M);
-        const int rt = m / rows_per_tile;
-        for (int i = ks; i < I; i += 4) {
-            const int first = (i * row_tiles + rt) * n_chunks;
-            const int nk = sp.owner(first + n_chunks - 1) - sp.owner(first) + 1;
-            const float *src = part + (((int64_t)i * kmax) * T + t) * M + m;
-            for (int k = 0; k < nk; k++) acc += src[(int64_t)k * T * M];
+    if (m < M) {
+        const int64_t stride = (int64_t)T * M;
+        for (int i = ks; i < I; i += RED_SL) {
+            const float *src = part + ((int64_t)i * kmax * T + t) * M + m;
+            const int nk = nks[i];
+            for (int k = 0; k < nk; k++) acc += src[k * stride];
         }
     }
     red[ks][lo] = acc;
     __syncthreads();
-    if (ks == 0 && o < total) {
-        float s = ((red[0][lo] + red[1][lo]) + red[2][lo]) + red[3][lo];
+    if (ks == 0 && m < M) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < RED_SL; k++) s += red[k][lo];
         if (bias) s += (float)bias[m];
-        y[o] = (half_t)s;
+        y[(int64_t)t * M + m] = (half_t)s;
     }
 }
 
@@ -488,6 +496,7 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
     if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 8)) return BS_ERR_SHAPE;
     const int64_t need = bs_gemv_workspace_bytes(I, M, N, K, T);
     if (!workspace || workspace_bytes < need) return BS_ERR_WORKSPACE;
+    if (I > RED_MAXBLOCKS) return BS_ERR_SHAPE;
     float *part = (float *)workspace;
     const int tp = pass_tokens(T);
     const Plan p = make_plan(I, M, N, tp);
@@ -502,8 +511,7 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
             default: st = launch_T<4>(p, packed, u, vt, xp, part, M, N, K, s); break;
         }
         if (st != BS_OK) return st;
-        const int64_t total = (int64_t)tn * M;
-        gemv_reduce_kernel<<<(int)bs_cdiv(total, 64), 256, 0, s>>>(part, bias, y + (int64_t)t0 * M, I, tn, M,
+        gemv_reduce_kernel<<<tn * (int)bs_cdiv(M, RED_OUT), RED_OUT * RED_SL, 0, s>>>(part, bias, y + (int64_t)t0 * M, I, tn, M,
                                                                    p.waves * p.R * 16, p.row_tiles, p.n_chunks,
                                                                    p.sp, p.kmax);
         BS_LAUNCH_CHECK();
