@@ -23,6 +23,8 @@ Extra objects on the same JSON line:
                 timed on this host on one pass of the same sweep.
   t4, prefill   the same sweep at 4 tokens, and the prefill configuration
                 (I = 8, T in {16, 128, 512, 2048}) as useful TFLOP/s.
+  decode_8b     tokens/s of a random-init Llama-3.1-8B-shape decode loop built
+                around the same forward (batch 1, 256 greedy tokens).
 """
 import argparse
 import json
@@ -94,6 +96,39 @@ def cpu_baseline(layers_cpu):
             "sample": f"the T=1 sweep restricted to blocks {{1,2,4}} on all four shapes ({len(layers_cpu)} layers, "
                       f"{tot_b / 1e6:.0f} MB algorithmic, {tot_t:.1f} s) through the level-0 torch-CPU restatement",
             "seconds": round(tot_t, 2)}
+
+
+def e2e_decode(torch, dev, prompt_len=128, new_tokens=256):
+    """Random-init Llama-3.1-8B-shape decode, batch 1: all 224 decoder linears are
+    BitStackLinear (level 5) with seeded per-layer block counts in [2, 12] summing
+    to about 5.5 GB with the dense embed / lm_head; one decode step is captured in a
+    HIP graph and replayed for `new_tokens` greedy tokens after a `prompt_len` prompt."""
+    from bitstack_amd.utils.llama_decode import LLAMA_8B, SyntheticLlamaDecoder, synthetic_compression_config
+    cfg, total = synthetic_compression_config(LLAMA_8B, 5.5e9)
+    model = SyntheticLlamaDecoder(LLAMA_8B, cfg, prompt_len + new_tokens + 8, dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        prompt = torch.randint(0, LLAMA_8B.vocab, (prompt_len,), generator=torch.Generator().manual_seed(0))
+        model.prefill_positions(prompt)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        model.step()
+    graph.replay()                       # the captured step also ran once during capture bookkeeping
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    wbytes = model.weight_bytes()
+    blocks = list(cfg.values())
+    return {"tok_s": round(new_tokens / dt, 1), "ms_per_token": round(dt / new_tokens * 1e3, 3),
+            "weight_GB": round(wbytes / 1e9, 3), "blocks_per_linear_mean": round(sum(blocks) / len(blocks), 2),
+            "hbm_roofline_tok_s": round(8e12 / wbytes, 1), "frac_of_hbm_roofline": round(new_tokens / dt * wbytes / 8e12, 4),
+            "config": f"32 layers, hidden 4096, inter 14336, 32Q/8KV, vocab 128256, batch 1, {prompt_len}-token prompt, "
+                      f"{new_tokens} greedy tokens, one HIP-graph replay per token"}
 
 
 def main():
@@ -193,10 +228,24 @@ def main():
     # (b) kernel time per forward from HIP events on the launch stream
     _, per_layer = time_sweep(layers, a.steps, 1, per_layer_events=True)
     ev_total_ms = sum(per_layer)
-    achieved = pass_bytes / (ev_total_ms * 1e-3) / 1e9
+    sweep_gbs = pass_bytes / (ev_total_ms * 1e-3) / 1e9
     detail = [{"M": L.M, "N": L.N, "I": L.I, "T": L.T, "bytes": L.bytes, "us": round(ms * 1e3, 2),
-               "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(layers, per_layer)]
+               "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1),
+               "kernel": "gemv_kernel<T=1,WAVES=%d,R=%d> x %d workgroups" % _lib.decode_plan(L.I, L.M, L.N, 16, 1)[:3]}
+              for L, ms in zip(layers, per_layer)]
     best = max(detail, key=lambda d: d["GBps"])
+    # dominant kernel = the instantiation that takes the most time over the pass
+    by_kernel = {}
+    for L, ms in zip(layers, per_layer):
+        key = "gemv_kernel<T=1,WAVES=%d,R=%d>" % _lib.decode_plan(L.I, L.M, L.N, 16, 1)[:2]
+        b, t, n = by_kernel.get(key, (0, 0.0, 0))
+        by_kernel[key] = (b + L.bytes, t + ms, n + 1)
+    dom, (dom_bytes, dom_ms, dom_n) = max(by_kernel.items(), key=lambda kv: kv[1][1])
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    # HBM bytes per forward measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the largest launch of
+    # that kernel (14336x4096, I=16), scaled by what the same counters read for a 256 MiB copy
+    # (FETCH_SIZE x2.0, WRITE_SIZE x1.0; profiles/gemv_traffic_counters.txt): 196 MB vs 126.9 MB algorithmic
+    traffic_ratio = 1.55
 
     out = {
         "metric": "packed-sign GEMV HBM GB/s (decode sweep, Llama-3.1-8B linear shapes, T=1)",
@@ -209,10 +258,15 @@ def main():
                    "launch": launch},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_kernel<T=1> + gemv_reduce_kernel per forward, HIP-event time summed over the sweep",
-                     "avg_us_per_forward": round(ev_total_ms * 1e3 / len(layers), 2),
-                     "avg_algorithmic_MB_per_forward": round(pass_bytes / len(layers) / 1e6, 3),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": round(dom_bytes / dom_n * traffic_ratio),
+                     "kernel": dom + " (+ its gemv_reduce_kernel), the instantiation with the most time in the pass",
+                     "launches_per_step": dom_n,
+                     "avg_us_per_launch": round(dom_ms * 1e3 / dom_n, 2),
+                     "avg_algorithmic_bytes_per_launch": round(dom_bytes / dom_n),
+                     "traffic_note": "HBM bytes per launch = algorithmic x 1.55, the FETCH_SIZE+WRITE_SIZE ratio "
+                                     "measured on this kernel's largest launch (profiles/gemv_traffic_counters.txt)",
+                     "whole_sweep_GBps_by_events": round(sweep_gbs, 1),
                      "best_layer": best},
     }
 
@@ -242,6 +296,9 @@ def main():
                        for L, ms in zip(lp, perp)]
             del lp
         out["prefill"] = pre
+
+    if not a.no_extras:
+        out["decode_8b"] = e2e_decode(torch, dev)
 
     if not a.no_cpu_baseline:
         # bounded sample of the same sweep: every shape, blocks {1, 2, 4} (7/31 of the pass)

@@ -26,6 +26,7 @@ SIGNATURES = {
     "bs_reconstruct_w_from_sign": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "bs_reconstruct_w": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "bs_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
+    "bs_decode_plan": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P]),
     "bs_forward": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _L, _P]),
     "bs_linear_f16": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
 }
@@ -56,6 +57,13 @@ def lib():
                     fn.restype, fn.argtypes = res, args
                 _lib = L
     return _lib
+
+
+def decode_plan(I, M, N, K, T):
+    """(waves, row_tiles_per_wave, workgroups, partials_per_row) of the decode kernel, waves == 0 if not used."""
+    vals = [ctypes.c_int(0) for _ in range(4)]
+    check(lib().bs_decode_plan(I, M, N, K, T, *[ctypes.byref(v) for v in vals]), "bs_decode_plan")
+    return tuple(v.value for v in vals)
 
 
 def error_string(status: int) -> str:

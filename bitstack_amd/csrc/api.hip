@@ -36,6 +36,15 @@ extern "C" int64_t bs_workspace_bytes(int I, int M, int N, int K, int T) {
     return round_up((int64_t)M * N * 2, 256);
 }
 
+extern "C" int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave,
+                              int *workgroups, int *partials_per_row) {
+    if (!waves || !row_tiles_per_wave || !workgroups || !partials_per_row) return BS_ERR_NULL;
+    int st = forward_dims(I, M, N, K, T);
+    if (st != BS_OK) return st;
+    bs_gemv_plan_info(I, M, N, T, waves, row_tiles_per_wave, workgroups, partials_per_row);
+    return BS_OK;
+}
+
 extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void *x,
                           const void *bias, void *y, int I, int M, int N, int K, int T,
                           void *workspace, int64_t workspace_bytes, void *stream) {

@@ -42,3 +42,4 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
                    const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
                    void *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T);
+void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax);

@@ -430,7 +430,9 @@ Plan make_plan(int I, int M, int N, int T) {
     p.row_tiles = (int)bs_cdiv(M, p.waves * p.R * 16);
     p.units = I * p.row_tiles * p.n_chunks;
     int grid = 256 * (T == 1 ? cand[pick][2] : T == 2 ? 2 : 1);
-    if (grid > p.units) grid = p.units;
+    // prefer two units per workgroup (one pipeline fill amortised over two units) as
+    // long as every CU still gets a workgroup
+    if (grid > p.units / 2) grid = p.units / 2 >= 256 ? p.units / 2 : (p.units < 256 ? p.units : 256);
     if (grid < 1) grid = 1;
     p.grid = grid;
     p.sp.q = p.units / grid;
@@ -485,6 +487,18 @@ int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T) {
     if (!gemv_shape_ok(I, M, N, T)) return 0;
     Plan p = make_plan(I, M, N, pass_tokens(T));
     return (int64_t)I * p.kmax * pass_tokens(T) * M * (int64_t)sizeof(float);
+}
+
+// Which instantiation and grid a decode forward of these dimensions runs
+// (0 in *waves when the decode kernel does not take them).
+void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax) {
+    *waves = *row_tiles_per_wave = *grid = *kmax = 0;
+    if (!gemv_shape_ok(I, M, N, T)) return;
+    const Plan p = make_plan(I, M, N, pass_tokens(T));
+    *waves = p.waves;
+    *row_tiles_per_wave = p.R;
+    *grid = p.grid;
+    *kmax = p.kmax;
 }
 
 // Returns BS_ERR_SHAPE when the fast path does not apply (the caller falls

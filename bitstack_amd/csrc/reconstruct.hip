@@ -2,37 +2,37 @@
 //   w[m, n] = fp16( sum_i s_i[m, n] * sum_r u_i[m, r] * vt_i[r, n] )
 // fp32 everywhere until the single final rounding.
 //
-// Tiled kernel: a workgroup owns 64 rows x 128 columns and walks the blocks.
-// Per block the rank-k product of a 16 x 16 patch is one MFMA
-// (v_mfma_f32_16x16x16_f16) computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
+// Tiled kernel.  A workgroup owns a strip of 128 columns and a range of rows.
+// It first stages the strip's slice of vt for ALL blocks in LDS, transposed to
+// [block][column][rank] (vt is stored rank-major, the MFMA wants the rank
+// index contiguous per lane; column stride 18 halves keeps the 8-byte fragment
+// reads off each other's banks), then walks its rows 16 per wave at a time with
+// no further barrier.  Per block the rank-k product of a 16 x 16 patch is one
+// v_mfma_f32_16x16x16_f16 computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
 // so that a lane ends up with four consecutive columns of one row - exactly
 // one nibble of that row's packed sign byte.  The sign is moved to bit 31,
-// merged into the constant 1.0f and applied with one FMA.
-//
-// vt is stored rank-major ([K, N]); the MFMA wants the rank index contiguous
-// per lane, so each block's 16 x 128 slice of vt goes through LDS transposed
-// (column stride 18 halves: 4-byte aligned reads, no bank aliasing between
-// the four 8-column pieces a wave writes at once).
+// merged into the constant 1.0f and applied with one FMA.  Signs and u of the
+// next block are loaded while the current block is multiplied.
 #include "common.h"
 
 namespace {
 
-constexpr int RT_ROWS = 64;    // rows per workgroup (16 per wave)
-constexpr int RT_COLS = 128;   // columns per workgroup
+constexpr int RT_COLS = 128;   // columns per workgroup strip
 constexpr int VSTRIDE = 18;    // halves between consecutive columns in LDS
+constexpr int RT_MAXB = 32;    // most blocks whose vt strip fits in LDS (32 x 4.5 KB)
 
 template <bool PACKED>
 __global__ __launch_bounds__(256) void reconstruct_tile_kernel(
     const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
     const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
-    int I, int M, int N, int K) {
-    __shared__ half_t vl[2][RT_COLS * VSTRIDE];
+    int I, int M, int N, int K, int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) half_t vl[];   // [I][RT_COLS][VSTRIDE]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * RT_COLS;
-    const int m0 = blockIdx.y * RT_ROWS + wave * 16;
-    const int row = min(m0 + lm, M - 1);
+    const int row_begin = blockIdx.y * rows_per_wg;
+    const int row_end = min(row_begin + rows_per_wg, M);
     const int64_t row_bytes = N >> 3;
     const int64_t block_bytes = (int64_t)M * row_bytes;
 
@@ -41,64 +41,80 @@ __global__ __launch_bounds__(256) void reconstruct_tile_kernel(
     // shift that brings this lane's first column of an even 16-column patch to bit 31
     const int sh_even = 24 - 8 * (g >> 1) + 4 * (g & 1);
 
-    float4_t acc[8];
+    {
+        const int i0 = 0, ib = I;
+        for (int i = 0; i < ib; i++) {
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (sr < K)
+                v = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
 #pragma unroll
-    for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-    for (int i = 0; i < I; i++) {
-        const int buf = i & 1;
-        half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (sr < K)
-            v = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
-#pragma unroll
-        for (int e = 0; e < 8; e++) vl[buf][(8 * sp + e) * VSTRIDE + sr] = v[e];
-
-        half4_t b;   // u_i[row, 4g .. 4g+3], zero beyond the rank
-        {
-            const half_t *up = u + ((int64_t)i * M + row) * K;
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[4 * g + j] : (half_t)0;
-        }
-
-        uint4_t sw = {0, 0, 0, 0};
-        if (PACKED) {
-            sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
-            sw = ~sw;   // bit 1 means +1: make it a clear IEEE sign bit
+            for (int e = 0; e < 8; e++) vl[(i * RT_COLS + 8 * sp + e) * VSTRIDE + sr] = v[e];
         }
         __syncthreads();
 
+        // 16 rows per wave and step
+        for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += 64) {
+            const int row = min(m0 + lm, M - 1);
+            float4_t acc[8];
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const half_t *ap = &vl[buf][(16 * s + lm) * VSTRIDE + 4 * g];
-            half2_t a01 = *reinterpret_cast<const half2_t *>(ap);
-            half2_t a23 = *reinterpret_cast<const half2_t *>(ap + 2);
-            half4_t a = {a01[0], a01[1], a23[0], a23[1]};
-            float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-            if (PACKED) {
-                uint32_t t = sw[s >> 1] << (sh_even - 16 * (s & 1));
+            for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+            auto load_block = [&](int i, half4_t &b, uint4_t &sw) {
+                const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+                if (K == 16) {
+                    b = *reinterpret_cast<const half4_t *>(up);
+                } else {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                    acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                    for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
                 }
-            } else {
-                uint32_t t = *reinterpret_cast<const uint32_t *>(
-                    sign + ((int64_t)i * M + row) * N + n0 + 16 * s + 4 * g);
+                if (PACKED) {
+                    sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
+                }
+            };
+
+            half4_t b_cur, b_nxt;
+            uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
+            load_block(i0, b_cur, sw_cur);
+            for (int i = 0; i < ib; i++) {
+                if (i + 1 < ib) load_block(i0 + i + 1, b_nxt, sw_nxt);
+                const uint4_t swc = ~sw_cur;     // bit 1 means +1: make it a clear IEEE sign bit
+                const half_t *vb = vl + (i * RT_COLS) * VSTRIDE;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
-                    acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                for (int s = 0; s < 8; s++) {
+                    const half_t *ap = vb + (16 * s + lm) * VSTRIDE + 4 * g;
+                    half2_t a01 = *reinterpret_cast<const half2_t *>(ap);
+                    half2_t a23 = *reinterpret_cast<const half2_t *>(ap + 2);
+                    half4_t a = {a01[0], a01[1], a23[0], a23[1]};
+                    float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    if (PACKED) {
+                        uint32_t t = swc[s >> 1] << (sh_even - 16 * (s & 1));
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
+                            acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                        }
+                    } else {
+                        uint32_t t = *reinterpret_cast<const uint32_t *>(
+                            sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 16 * s + 4 * g);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
+                            acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                        }
+                    }
+                }
+                b_cur = b_nxt;
+                sw_cur = sw_nxt;
+            }
+
+            if (m0 + lm < M) {
+                half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 4 * g;
+#pragma unroll
+                for (int s = 0; s < 8; s++) {
+                    half4_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
+                    *reinterpret_cast<half4_t *>(wp + 16 * s) = o;
                 }
             }
-        }
-    }
-
-    if (m0 + lm < M) {
-        half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 4 * g;
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            half4_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-            *reinterpret_cast<half4_t *>(wp + 16 * s) = o;
         }
     }
 }
@@ -136,11 +152,25 @@ __global__ __launch_bounds__(256) void reconstruct_generic_kernel(
 template <bool PACKED>
 int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *u, const half_t *vt,
                        half_t *w, int I, int M, int N, int K, hipStream_t s) {
-    const bool tiled = (N % RT_COLS == 0) && bs_aligned(vt, 16) && bs_aligned(w, 8) &&
-                       (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
+    const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && bs_aligned(vt, 16) && bs_aligned(w, 8) &&
+                       bs_aligned(u, 8) && (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
     if (tiled) {
-        dim3 grid(N / RT_COLS, (unsigned)bs_cdiv(M, RT_ROWS));
-        reconstruct_tile_kernel<PACKED><<<grid, 256, 0, s>>>(packed, sign, u, vt, w, I, M, N, K);
+        // about four workgroups per CU; every workgroup re-stages its vt strip, so rows
+        // per workgroup stay a multiple of 64 and not too small
+        const int strips = N / RT_COLS;
+        int row_groups = (int)bs_cdiv(1024, strips);
+        int rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
+        if (rows_per_wg < 128) rows_per_wg = 128;
+        row_groups = (int)bs_cdiv(M, rows_per_wg);
+        const size_t lds = (size_t)I * RT_COLS * VSTRIDE * sizeof(half_t);
+        static size_t raised = 0;
+        if (lds > 64 * 1024 && lds > raised) {
+            BS_HIP_TRY(hipFuncSetAttribute((const void *)reconstruct_tile_kernel<PACKED>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            raised = lds;
+        }
+        dim3 grid(strips, row_groups);
+        reconstruct_tile_kernel<PACKED><<<grid, 256, lds, s>>>(packed, sign, u, vt, w, I, M, N, K, rows_per_wg);
     } else {
         int64_t blocks = bs_cdiv((int64_t)M * N, 256);
         if (blocks > 256 * 64) blocks = 256 * 64;

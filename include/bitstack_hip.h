@@ -105,6 +105,18 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
                void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Introspection for benchmarks and tests: which decode kernel instantiation
+ * (waves per workgroup, 16-row tiles per wave), how many workgroups and how
+ * many partial sums per row and block bs_forward would use for these
+ * dimensions; *waves == 0 means the decode kernel does not take them (more
+ * than 8 tokens, N not a multiple of 512).  No counterpart in the reference
+ * (Triton picks its configuration by autotuning,
+ * bitstack/utils/inference_utils.py:8-39).
+ */
+int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave,
+                   int *workgroups, int *partials_per_row);
+
+/*
  * y[T, M] = x[T, N] @ w[M, N]^T (+ bias) on MFMA, fp32 accumulation: the
  * dense contraction bs_forward uses for large T, exposed for levels 2-4 where
  * the reference calls F.linear on the rebuilt weight
