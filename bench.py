@@ -102,29 +102,40 @@ def e2e_decode(torch, dev, prompt_len=128, new_tokens=256):
     """Random-init Llama-3.1-8B-shape decode, batch 1: all 224 decoder linears are
     BitStackLinear (level 5) with seeded per-layer block counts in [2, 12] summing
     to about 5.5 GB with the dense embed / lm_head; one decode step is captured in a
-    HIP graph and replayed for `new_tokens` greedy tokens after a `prompt_len` prompt."""
+    HIP graph and replayed for `new_tokens` greedy tokens after a `prompt_len` prompt.
+    Measured twice: the fused step (grouped forwards + the library's RMSNorm and
+    attention kernels; the headline) and the step with one call per linear and
+    torch ops in between."""
     from bitstack_amd.utils.llama_decode import LLAMA_8B, SyntheticLlamaDecoder, synthetic_compression_config
     cfg, total = synthetic_compression_config(LLAMA_8B, 5.5e9)
     model = SyntheticLlamaDecoder(LLAMA_8B, cfg, prompt_len + new_tokens + 8, dev)
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        prompt = torch.randint(0, LLAMA_8B.vocab, (prompt_len,), generator=torch.Generator().manual_seed(0))
-        model.prefill_positions(prompt)
-    side.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        model.step()
-    graph.replay()                       # the captured step also ran once during capture bookkeeping
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(new_tokens):
-        graph.replay()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    prompt = torch.randint(0, LLAMA_8B.vocab, (prompt_len,), generator=torch.Generator().manual_seed(0))
+
+    def run(fused):
+        step = model.step_fused if fused else model.step
+        model.reset()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.prefill_positions(prompt, fused=fused)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        graph.replay()                   # the captured step also ran once during capture bookkeeping
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(new_tokens):
+            graph.replay()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    dt_plain = run(False)
+    dt = run(True)
     wbytes = model.weight_bytes()
     blocks = list(cfg.values())
     return {"tok_s": round(new_tokens / dt, 1), "ms_per_token": round(dt / new_tokens * 1e3, 3),
+            "tok_s_one_call_per_linear_torch_ops_between": round(new_tokens / dt_plain, 1),
             "weight_GB": round(wbytes / 1e9, 3), "blocks_per_linear_mean": round(sum(blocks) / len(blocks), 2),
             "hbm_roofline_tok_s": round(8e12 / wbytes, 1), "frac_of_hbm_roofline": round(new_tokens / dt * wbytes / 8e12, 4),
             "config": f"32 layers, hidden 4096, inter 14336, 32Q/8KV, vocab 128256, batch 1, {prompt_len}-token prompt, "

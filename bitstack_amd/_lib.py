@@ -31,6 +31,21 @@ SIGNATURES = {
     "bs_linear_f16": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
 }
 
+
+
+class bs_matrix(ctypes.Structure):
+    """struct bs_matrix of include/bitstack_hip.h."""
+    _fields_ = [("packed", _P), ("u", _P), ("vt", _P), ("bias", _P), ("I", ctypes.c_int32), ("M", ctypes.c_int32)]
+
+
+SIGNATURES.update({
+    "bs_forward_group_workspace_bytes": (_L, [_P, _I, _I, _I, _I]),
+    "bs_forward_group": (_I, [_P, _I, _I, _I, _P, _I, _I, _P, _P, _P, _L, _P]),
+    "bs_rmsnorm_f16": (_I, [_P, _P, _P, _I, _I, ctypes.c_float, _P]),
+    "bs_attention_decode_f16": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+})
+EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU = 0, 1, 2
+
 _lib = None
 _lock = threading.Lock()
 

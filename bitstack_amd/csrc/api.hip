@@ -71,3 +71,80 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     if (st != BS_OK) return st;
     return bs_launch_linear_f16((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N, s);
 }
+
+// ---- grouped decode forward ---------------------------------------------------
+static int group_dims(const bs_matrix *mats, int n, int N, int K, int T) {
+    if (!mats) return BS_ERR_NULL;
+    if (n < 1 || n > BS_MAX_GROUP) return BS_ERR_SHAPE;
+    for (int j = 0; j < n; j++) {
+        int st = forward_dims(mats[j].I, mats[j].M, N, K, T);
+        if (st != BS_OK) return st;
+        if (mats[j].I < 1) return BS_ERR_SHAPE;
+    }
+    if (T < 1 || T > 8) return BS_ERR_SHAPE;
+    return BS_OK;
+}
+
+extern "C" int64_t bs_forward_group_workspace_bytes(const bs_matrix *mats, int n, int N, int K, int T) {
+    int st = group_dims(mats, n, N, K, T);
+    if (st != BS_OK) return st;
+    int I[BS_MAX_GROUP], M[BS_MAX_GROUP];
+    for (int j = 0; j < n; j++) { I[j] = mats[j].I; M[j] = mats[j].M; }
+    const int64_t b = bs_gemv_group_workspace_bytes(I, M, n, N, K, T);
+    return b > 0 ? round_up(b, 256) : (int64_t)BS_ERR_SHAPE;
+}
+
+extern "C" int bs_forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, int T,
+                                int epilogue, const void *residual, void *y,
+                                void *workspace, int64_t workspace_bytes, void *stream) {
+    int st = group_dims(mats, n, N, K, T);
+    if (st != BS_OK) return st;
+    if (epilogue != BS_EPI_NONE && epilogue != BS_EPI_RESIDUAL && epilogue != BS_EPI_SWIGLU) return BS_ERR_SHAPE;
+    if (!x || !y || (epilogue == BS_EPI_RESIDUAL && !residual)) return BS_ERR_NULL;
+    const uint8_t *packed[BS_MAX_GROUP];
+    const half_t *u[BS_MAX_GROUP], *vt[BS_MAX_GROUP], *bias[BS_MAX_GROUP];
+    int I[BS_MAX_GROUP], M[BS_MAX_GROUP];
+    for (int j = 0; j < n; j++) {
+        if (!mats[j].packed || !mats[j].u || !mats[j].vt) return BS_ERR_NULL;
+        if (!bs_aligned(mats[j].packed, 16) || !bs_aligned(mats[j].vt, 16) || !bs_aligned(mats[j].u, 8) ||
+            !bs_aligned(mats[j].bias, 2))
+            return BS_ERR_ALIGN;
+        packed[j] = mats[j].packed;
+        u[j] = (const half_t *)mats[j].u;
+        vt[j] = (const half_t *)mats[j].vt;
+        bias[j] = (const half_t *)mats[j].bias;
+        I[j] = mats[j].I;
+        M[j] = mats[j].M;
+    }
+    if (!bs_aligned(x, 16) || !bs_aligned(y, 2) || !bs_aligned(residual, 2)) return BS_ERR_ALIGN;
+    const int64_t need = bs_forward_group_workspace_bytes(mats, n, N, K, T);
+    if (need < 0) return (int)need;
+    if (!workspace || workspace_bytes < need || !bs_aligned(workspace, 256)) return BS_ERR_WORKSPACE;
+    return bs_launch_gemv_group(n, packed, u, vt, bias, I, M, N, K, (const half_t *)x, T, epilogue,
+                                (const half_t *)residual, (half_t *)y, workspace, workspace_bytes,
+                                (hipStream_t)stream);
+}
+
+extern "C" int bs_rmsnorm_f16(const void *x, const void *weight, void *y, int T, int H, float eps, void *stream) {
+    if (T < 0 || H <= 0 || H % 8 != 0 || H > 16384) return BS_ERR_SHAPE;
+    if (T == 0) return BS_OK;
+    if (!x || !weight || !y) return BS_ERR_NULL;
+    if (!bs_aligned(x, 16) || !bs_aligned(weight, 16) || !bs_aligned(y, 16)) return BS_ERR_ALIGN;
+    return bs_launch_rmsnorm((const half_t *)x, (const half_t *)weight, (half_t *)y, T, H, eps, (hipStream_t)stream);
+}
+
+extern "C" int bs_attention_decode_f16(const void *qkv, void *kcache, void *vcache, const void *cos, const void *sin,
+                                       const int64_t *pos, void *out, int B, int heads, int kv_heads, int head_dim,
+                                       int max_len, void *stream) {
+    if (B < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim != 128 || max_len < 1 ||
+        max_len > 8192)
+        return BS_ERR_SHAPE;
+    if (B == 0) return BS_OK;
+    if (!qkv || !kcache || !vcache || !cos || !sin || !pos || !out) return BS_ERR_NULL;
+    if (!bs_aligned(qkv, 16) || !bs_aligned(kcache, 16) || !bs_aligned(vcache, 16) || !bs_aligned(cos, 16) ||
+        !bs_aligned(sin, 16) || !bs_aligned(pos, 8) || !bs_aligned(out, 16))
+        return BS_ERR_ALIGN;
+    return bs_launch_attention_decode((const half_t *)qkv, (half_t *)kcache, (half_t *)vcache, (const half_t *)cos,
+                                      (const half_t *)sin, pos, (half_t *)out, B, heads, kv_heads, head_dim, max_len,
+                                      (hipStream_t)stream);
+}

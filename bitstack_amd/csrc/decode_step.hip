@@ -1,0 +1,175 @@
+// The two steps of a decoder layer that sit between the compressed linears at
+// decode time: RMSNorm, and one position of rotary grouped-query attention over a
+// static KV cache.  Small, latency-bound kernels; their point is to replace a
+// dozen framework launches per layer by two.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// One workgroup per row; the row stays in registers between the two passes.
+constexpr int RMS_THREADS = 256, RMS_MAX_CHUNKS = 8;   // 256 * 8 * 8 halves = 16384 columns
+
+__global__ __launch_bounds__(RMS_THREADS) void rmsnorm_kernel(const half_t *__restrict__ x,
+                                                              const half_t *__restrict__ weight,
+                                                              half_t *__restrict__ y, int H, float eps) {
+    __shared__ float wsum[RMS_THREADS / 64];
+    const int tid = threadIdx.x;
+    const half_t *xr = x + (int64_t)blockIdx.x * H;
+    half_t *yr = y + (int64_t)blockIdx.x * H;
+    half8_t v[RMS_MAX_CHUNKS];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < RMS_MAX_CHUNKS; c++) {
+        const int col = (c * RMS_THREADS + tid) * 8;
+        if (col < H) {
+            v[c] = *reinterpret_cast<const half8_t *>(xr + col);
+#pragma unroll
+            for (int e = 0; e < 8; e++) ss += (float)v[c][e] * (float)v[c][e];
+        }
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) wsum[tid >> 6] = ss;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < RMS_THREADS / 64; w++) total += wsum[w];
+    const float r = rsqrtf(total / (float)H + eps);
+#pragma unroll
+    for (int c = 0; c < RMS_MAX_CHUNKS; c++) {
+        const int col = (c * RMS_THREADS + tid) * 8;
+        if (col < H) {
+            const half8_t w8 = *reinterpret_cast<const half8_t *>(weight + col);
+            half8_t o;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = (half_t)((float)(half_t)((float)v[c][e] * r) * (float)w8[e]);
+            *reinterpret_cast<half8_t *>(yr + col) = o;
+        }
+    }
+}
+
+// One workgroup per (query head, sequence).  256 threads = 16 groups of 16 lanes;
+// a group walks every 16th cached position, a lane owns 8 of the 128 dimensions
+// (one 16-byte load per cached row and lane, a row is one contiguous 256 bytes).
+constexpr int ATT_THREADS = 256, ATT_D = 128, ATT_MAX_LEN = 8192;
+
+__global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
+    const half_t *__restrict__ qkv, half_t *__restrict__ kcache, half_t *__restrict__ vcache,
+    const half_t *__restrict__ cosv, const half_t *__restrict__ sinv, const int64_t *__restrict__ pos_ptr,
+    half_t *__restrict__ out, int heads, int kv_heads, int max_len) {
+    __shared__ float score[ATT_MAX_LEN];
+    __shared__ float qs[ATT_D];                  // rotated query, pre-scaled
+    __shared__ __attribute__((aligned(16))) half_t knew[ATT_D], vnew[ATT_D];   // this position's rotated k and v
+    __shared__ float red[ATT_THREADS / 64];
+    __shared__ float accs[16][ATT_D];
+    const int tid = threadIdx.x, lane16 = tid & 15, grp = tid >> 4;
+    const int head = blockIdx.x, b = blockIdx.y;
+    const int rep = heads / kv_heads, hk = head / rep;
+    const int row = (heads + 2 * kv_heads) * ATT_D;
+    const half_t *q = qkv + (int64_t)b * row + head * ATT_D;
+    const half_t *kn = qkv + (int64_t)b * row + (heads + hk) * ATT_D;
+    const half_t *vn = qkv + (int64_t)b * row + (heads + kv_heads + hk) * ATT_D;
+    half_t *orow = out + ((int64_t)b * heads + head) * ATT_D;
+    const int64_t pos64 = *pos_ptr;
+    if (pos64 < 0 || pos64 >= max_len) {         // nothing sensible to do: defined output, no access outside the cache
+        if (tid < ATT_D) orow[tid] = (half_t)0;
+        return;
+    }
+    const int pos = (int)pos64;
+    half_t *kc = kcache + ((int64_t)b * kv_heads + hk) * max_len * ATT_D;
+    half_t *vc = vcache + ((int64_t)b * kv_heads + hk) * max_len * ATT_D;
+
+    if (tid < ATT_D / 2) {
+        const float c = (float)cosv[(int64_t)pos * (ATT_D / 2) + tid], s = (float)sinv[(int64_t)pos * (ATT_D / 2) + tid];
+        const float qa = (float)q[tid], qb = (float)q[tid + ATT_D / 2];
+        const float scale = 0.08838834764831845f;       // 1 / sqrt(128)
+        qs[tid] = (float)(half_t)(qa * c - qb * s) * scale;
+        qs[tid + ATT_D / 2] = (float)(half_t)(qb * c + qa * s) * scale;
+        const float ka = (float)kn[tid], kb = (float)kn[tid + ATT_D / 2];
+        knew[tid] = (half_t)(ka * c - kb * s);
+        knew[tid + ATT_D / 2] = (half_t)(kb * c + ka * s);
+    } else if (tid < ATT_D / 2 + ATT_D) {
+        vnew[tid - ATT_D / 2] = vn[tid - ATT_D / 2];
+    }
+    __syncthreads();
+    if (head % rep == 0 && tid < ATT_D) {        // one head of the group appends to the cache
+        kc[(int64_t)pos * ATT_D + tid] = knew[tid];
+        vc[(int64_t)pos * ATT_D + tid] = vnew[tid];
+    }
+
+    float qreg[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) qreg[e] = qs[8 * lane16 + e];
+    for (int p = grp; p <= pos; p += 16) {
+        const half8_t k8 = p == pos ? *reinterpret_cast<const half8_t *>(knew + 8 * lane16)
+                                    : *reinterpret_cast<const half8_t *>(kc + (int64_t)p * ATT_D + 8 * lane16);
+        float d = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) d += qreg[e] * (float)k8[e];
+#pragma unroll
+        for (int o = 8; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
+        if (lane16 == 0) score[p] = d;
+    }
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int p = tid; p <= pos; p += ATT_THREADS) mx = fmaxf(mx, score[p]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.f;
+    for (int p = tid; p <= pos; p += ATT_THREADS) {
+        const float e = __expf(score[p] - mx);
+        score[p] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if ((tid & 63) == 0) red[tid >> 6] = sum;
+    __syncthreads();
+    const float inv = 1.f / (red[0] + red[1] + red[2] + red[3]);
+
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int p = grp; p <= pos; p += 16) {
+        const half8_t v8 = p == pos ? *reinterpret_cast<const half8_t *>(vnew + 8 * lane16)
+                                    : *reinterpret_cast<const half8_t *>(vc + (int64_t)p * ATT_D + 8 * lane16);
+        const float w = (float)(half_t)(score[p] * inv);      // probabilities rounded to fp16 before the product
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += w * (float)v8[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) accs[grp][8 * lane16 + e] = acc[e];
+    __syncthreads();
+    if (tid < ATT_D) {
+        float o = 0.f;
+#pragma unroll
+        for (int gq = 0; gq < 16; gq++) o += accs[gq][tid];
+        orow[tid] = (half_t)o;
+    }
+}
+
+}  // namespace
+
+int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s) {
+    if (H > RMS_THREADS * RMS_MAX_CHUNKS * 8) return BS_ERR_SHAPE;
+    rmsnorm_kernel<<<T, RMS_THREADS, 0, s>>>(x, weight, y, H, eps);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
+int bs_launch_attention_decode(const half_t *qkv, half_t *kcache, half_t *vcache, const half_t *cos, const half_t *sin,
+                               const int64_t *pos, half_t *out, int B, int heads, int kv_heads, int head_dim,
+                               int max_len, hipStream_t s) {
+    if (head_dim != ATT_D || max_len > ATT_MAX_LEN) return BS_ERR_SHAPE;
+    attention_decode_kernel<<<dim3(heads, B), ATT_THREADS, 0, s>>>(qkv, kcache, vcache, cos, sin, pos, out, heads,
+                                                                  kv_heads, max_len);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}

@@ -126,11 +126,25 @@ struct Split {
     }
 };
 
+// Up to GEMV_MAX_GROUP matrices that share x (and so N and K) run in one launch:
+// the grid is cut into one run of workgroups per matrix, each with its own static
+// partition, partial-sum area and row count.
+constexpr int GEMV_MAX_GROUP = 4;
+struct GemvMat {
+    const uint8_t *packed;
+    const half_t *u, *vt;
+    float *part;
+    int M, row_tiles, kmax, first_wg;
+    Split sp;
+};
+struct GemvGroup {
+    GemvMat m[GEMV_MAX_GROUP];
+    int n;
+};
+
 template <int T, int WAVES, int R>
 __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? 2 : 1))) void gemv_kernel(
-    const uint8_t *__restrict__ packed, const half_t *__restrict__ u, const half_t *__restrict__ vt,
-    const half_t *__restrict__ x, float *__restrict__ part,
-    int M, int N, int K, int row_tiles, int n_chunks, Split sp, int kmax) {
+    const GemvGroup grp, const half_t *__restrict__ x, int N, int K, int n_chunks) {
     constexpr int RW = WAVES * R * 16;          // rows per workgroup
     constexpr int COMBOS = 8 / WAVES;           // (jb, pg) producer combos per wave
     constexpr int ZHALVES = T * 16 * 4 * 16 * 8;   // one Z buffer
@@ -151,6 +165,18 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
         const int base = nb >> 3, rem = nb & 7;
         wg = xcd * base + min(xcd, rem) + loc;
     }
+    // which matrix this workgroup belongs to (all of it is wave-uniform)
+    GemvMat mat = grp.m[0];
+#pragma unroll
+    for (int j = 1; j < GEMV_MAX_GROUP; j++)
+        if (j < grp.n && wg >= grp.m[j].first_wg) mat = grp.m[j];
+    wg -= mat.first_wg;
+    const uint8_t *__restrict__ packed = mat.packed;
+    const half_t *__restrict__ u = mat.u;
+    const half_t *__restrict__ vt = mat.vt;
+    float *__restrict__ part = mat.part;
+    const int M = mat.M, row_tiles = mat.row_tiles, kmax = mat.kmax;
+    const Split sp = mat.sp;
     const int u_begin = sp.start(wg), u_end = sp.start(wg + 1);
     if (u_begin >= u_end) return;
 
@@ -365,56 +391,108 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     if (warm == 0x9e3779b9u && part == nullptr) part[0] = 0.f;   // keeps the warm-up loads alive
 }
 
-// y[t, m] = fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) where k runs over the
-// workgroups whose unit range touched (block i, row tile of m), in ascending
-// order.  32 outputs of one row tile per workgroup; the number of partials of
-// every block is worked out once (one thread per block) into LDS, eight
-// threads per output take every eighth block (their loads are independent)
+// y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ) where k
+// runs over the workgroups whose unit range touched (block i, row tile of m), in
+// ascending order.  32 outputs of one row tile per workgroup; the number of
+// partials of every block is worked out once (one thread per block) into LDS,
+// eight threads per output take every eighth block (their loads are independent)
 // and are combined through LDS in a fixed order.
+// Epilogues (applied to the fp16-rounded sums, the way separate fp16 ops would):
+//   EPI_NONE      the matrices' outputs side by side in one row of `ldy` halves
+//   EPI_RESIDUAL  the same plus residual[t, off + m]
+//   EPI_SWIGLU    two matrices of equal M: silu(first) * second, one row of M
 constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;
 
-__global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
-    const float *__restrict__ part, const half_t *__restrict__ bias, half_t *__restrict__ y,
-    int I, int T, int M, int rows_per_tile, int row_tiles, int n_chunks, Split sp, int kmax) {
-    __shared__ int nks[RED_MAXBLOCKS];           // live partials of block i for this row tile
-    __shared__ float red[RED_SL][RED_OUT];
+struct RedMat {
+    const float *part;
+    const half_t *bias;
+    int I, M, row_tiles, kmax, y_off, first_block;
+    Split sp;
+};
+struct RedGroup {
+    RedMat m[GEMV_MAX_GROUP];
+    int n, mode;
+};
+
+__device__ __forceinline__ float reduce_partials(const RedMat &r, int T, int t, int m0, int rows_per_tile, int n_chunks,
+                                                 int *nks, float (*red)[RED_OUT]) {
     const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
-    // outputs are enumerated per token in runs of RED_OUT rows, so a workgroup never straddles tokens
-    const int per_t = (M + RED_OUT - 1) / RED_OUT;
-    const int t = blockIdx.x / per_t, m0 = (blockIdx.x - t * per_t) * RED_OUT, m = m0 + lo;
+    const int m = m0 + lo;
     const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
-    for (int i = threadIdx.x; i < I; i += RED_OUT * RED_SL) {
-        const int first = (i * row_tiles + rt) * n_chunks;
-        nks[i] = sp.owner(first + n_chunks - 1) - sp.owner(first) + 1;
+    for (int i = threadIdx.x; i < r.I; i += RED_OUT * RED_SL) {
+        const int first = (i * r.row_tiles + rt) * n_chunks;
+        nks[i] = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
     }
     __syncthreads();
     float acc = 0.f;
-    if (m < M) {
-        const int64_t stride = (int64_t)T * M;
-        for (int i = ks; i < I; i += RED_SL) {
-            const float *src = part + ((int64_t)i * kmax * T + t) * M + m;
+    if (m < r.M) {
+        const int64_t stride = (int64_t)T * r.M;
+        for (int i = ks; i < r.I; i += RED_SL) {
+            const float *src = r.part + ((int64_t)i * r.kmax * T + t) * r.M + m;
             const int nk = nks[i];
             for (int k = 0; k < nk; k++) acc += src[k * stride];
         }
     }
     red[ks][lo] = acc;
     __syncthreads();
-    if (ks == 0 && m < M) {
-        float s = 0.f;
+    float s = 0.f;
+    if (ks == 0 && m < r.M) {
 #pragma unroll
         for (int k = 0; k < RED_SL; k++) s += red[k][lo];
-        if (bias) s += (float)bias[m];
-        y[(int64_t)t * M + m] = (half_t)s;
+        if (r.bias) s += (float)r.bias[m];
+    }
+    __syncthreads();                             // nks / red are reused by a second call
+    return s;
+}
+
+__global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
+    const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy,
+    int rows_per_tile, int n_chunks) {
+    __shared__ int nks[RED_MAXBLOCKS];           // live partials of block i for this row tile
+    __shared__ float red[RED_SL][RED_OUT];
+    const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
+    int j = 0;
+    if (grp.mode != EPI_SWIGLU) {
+#pragma unroll
+        for (int q = 1; q < GEMV_MAX_GROUP; q++)
+            if (q < grp.n && (int)blockIdx.x >= grp.m[q].first_block) j = q;
+    }
+    const RedMat &r = grp.m[j];
+    // outputs are enumerated per token in runs of RED_OUT rows, so a workgroup never straddles tokens
+    const int local = blockIdx.x - r.first_block;
+    const int per_t = (r.M + RED_OUT - 1) / RED_OUT;
+    const int t = local / per_t, m0 = (local - t * per_t) * RED_OUT, m = m0 + lo;
+    const float s0 = reduce_partials(r, T, t, m0, rows_per_tile, n_chunks, nks, red);
+    if (grp.mode == EPI_SWIGLU) {
+        const float s1 = reduce_partials(grp.m[1], T, t, m0, rows_per_tile, n_chunks, nks, red);
+        if (ks == 0 && m < r.M) {
+            const float gate = (float)(half_t)s0, up = (float)(half_t)s1;
+            const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
+            y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
+        }
+        return;
+    }
+    if (ks == 0 && m < r.M) {
+        const int64_t at = (int64_t)t * ldy + r.y_off + m;
+        half_t v = (half_t)s0;
+        if (grp.mode == EPI_RESIDUAL) v = (half_t)((float)residual[at] + (float)v);
+        y[at] = v;
     }
 }
 
 struct Plan {
-    int waves, R, row_tiles, n_chunks, units, grid, kmax;
-    Split sp;
+    int waves, R, n_chunks, grid, n;
+    int row_tiles[GEMV_MAX_GROUP], kmax[GEMV_MAX_GROUP], first_wg[GEMV_MAX_GROUP];
+    Split sp[GEMV_MAX_GROUP];
+    int64_t part_off[GEMV_MAX_GROUP];      // in floats; part_off[n] = total
+    int64_t part_total;
 };
 
-Plan make_plan(int I, int M, int N, int T) {
+// One instantiation and one grid for the whole group; every matrix gets a share of
+// the workgroups in proportion to its units.
+Plan make_plan(const int *I, const int *M, int n, int N, int T) {
     Plan p;
+    p.n = n;
     p.n_chunks = N / CH;
     // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU
     const int cand[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
@@ -422,31 +500,59 @@ Plan make_plan(int I, int M, int N, int T) {
     // three or four tokens need more than the 256 registers an 8-wave workgroup can have
     for (int k = (T > 2 ? 1 : 0); k < 4; k++) {
         const int rw = cand[k][0] * cand[k][1] * 16;
+        bool tall = true;
+        int64_t units = 0;
+        for (int j = 0; j < n; j++) {
+            tall = tall && M[j] >= rw;
+            units += bs_cdiv(M[j], rw) * I[j] * p.n_chunks;
+        }
         // enough units that every CU gets one
-        if (M >= rw && bs_cdiv(M, rw) * I * p.n_chunks >= 256) { pick = k; break; }
+        if (tall && units >= 256) { pick = k; break; }
     }
     p.waves = cand[pick][0];
     p.R = cand[pick][1];
-    p.row_tiles = (int)bs_cdiv(M, p.waves * p.R * 16);
-    p.units = I * p.row_tiles * p.n_chunks;
+    int units[GEMV_MAX_GROUP], total = 0;
+    for (int j = 0; j < n; j++) {
+        p.row_tiles[j] = (int)bs_cdiv(M[j], p.waves * p.R * 16);
+        units[j] = I[j] * p.row_tiles[j] * p.n_chunks;
+        total += units[j];
+    }
     int grid = 256 * (T == 1 ? cand[pick][2] : T == 2 ? 2 : 1);
     // prefer two units per workgroup (one pipeline fill amortised over two units) as
     // long as every CU still gets a workgroup
-    if (grid > p.units / 2) grid = p.units / 2 >= 256 ? p.units / 2 : (p.units < 256 ? p.units : 256);
+    if (grid > total / 2) grid = total / 2 >= 256 ? total / 2 : (total < 256 ? total : 256);
     if (grid < 1) grid = 1;
-    p.grid = grid;
-    p.sp.q = p.units / grid;
-    p.sp.rem = p.units % grid;
-    // most workgroups a row of n_chunks units can be spread over
-    int kmax = (int)bs_cdiv(p.n_chunks - 1, p.sp.q) + 1;
-    if (kmax > grid) kmax = grid;
-    p.kmax = kmax;
+    int first = 0;
+    int64_t off = 0;
+    for (int j = 0; j < n; j++) {
+        int gj = n == 1 ? grid : (int)(((int64_t)grid * units[j] + total / 2) / total);
+        if (gj < 1) gj = 1;
+        if (gj > units[j]) gj = units[j];
+        p.first_wg[j] = first;
+        first += gj;
+        p.sp[j].q = units[j] / gj;
+        p.sp[j].rem = units[j] % gj;
+        // most workgroups a row of n_chunks units can be spread over
+        int kmax = (int)bs_cdiv(p.n_chunks - 1, p.sp[j].q) + 1;
+        if (kmax > gj) kmax = gj;
+        p.kmax[j] = kmax;
+        p.part_off[j] = off;
+        off += (int64_t)I[j] * kmax * T * M[j];
+    }
+    p.grid = first;
+    p.part_total = off;
     return p;
 }
 
+struct GroupArgs {          // host-side view of one call
+    int n;
+    const uint8_t *packed[GEMV_MAX_GROUP];
+    const half_t *u[GEMV_MAX_GROUP], *vt[GEMV_MAX_GROUP], *bias[GEMV_MAX_GROUP];
+    int I[GEMV_MAX_GROUP], M[GEMV_MAX_GROUP];
+};
+
 template <int T, int WAVES, int R>
-int launch_one(const Plan &p, const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-               float *part, int M, int N, int K, hipStream_t s) {
+int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     const size_t lds = (size_t)2 * T * 16384 + (size_t)2 * WAVES * T * 64;
     static bool raised = false;      // per instantiation; raising the limit is idempotent
     if (lds > 64 * 1024 && !raised) {
@@ -454,39 +560,107 @@ int launch_one(const Plan &p, const uint8_t *packed, const half_t *u, const half
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    gemv_kernel<T, WAVES, R><<<p.grid, 64 * WAVES, lds, s>>>(packed, u, vt, x, part, M, N, K, p.row_tiles,
-                                                            p.n_chunks, p.sp, p.kmax);
+    gemv_kernel<T, WAVES, R><<<p.grid, 64 * WAVES, lds, s>>>(grp, x, N, K, p.n_chunks);
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
 
 template <int T>
-int launch_T(const Plan &p, const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-             float *part, int M, int N, int K, hipStream_t s) {
+int launch_T(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     if (p.waves == 8) {
-        if constexpr (T <= 2) return launch_one<T, 8, 4>(p, packed, u, vt, x, part, M, N, K, s);
+        if constexpr (T <= 2) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
         else return BS_ERR_SHAPE;     // the planner never pairs 8 waves with more than two tokens
     }
-    if (p.R == 4) return launch_one<T, 4, 4>(p, packed, u, vt, x, part, M, N, K, s);
-    if (p.R == 2) return launch_one<T, 4, 2>(p, packed, u, vt, x, part, M, N, K, s);
-    return launch_one<T, 4, 1>(p, packed, u, vt, x, part, M, N, K, s);
+    if (p.R == 4) return launch_one<T, 4, 4>(p, grp, x, N, K, s);
+    if (p.R == 2) return launch_one<T, 4, 2>(p, grp, x, N, K, s);
+    return launch_one<T, 4, 1>(p, grp, x, N, K, s);
+}
+
+bool gemv_shape_ok(int I, int M, int N, int T) {
+    // per-block byte offsets are kept in 32 bits inside the kernel
+    return I >= 1 && I <= RED_MAXBLOCKS && T >= 1 && T <= 8 && N % CH == 0 && M >= 1 &&
+           (int64_t)M * N < ((int64_t)1 << 31);
+}
+
+// Tokens are processed in passes of at most four (LDS holds Z for four tokens).
+int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
+
+int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int mode, const half_t *residual,
+                 half_t *y, void *workspace, int64_t workspace_bytes, hipStream_t s) {
+    if (a.n < 1 || a.n > GEMV_MAX_GROUP) return BS_ERR_SHAPE;
+    if (!bs_aligned(x, 16)) return BS_ERR_SHAPE;
+    int ldy = 0;
+    for (int j = 0; j < a.n; j++) {
+        if (!gemv_shape_ok(a.I[j], a.M[j], N, T)) return BS_ERR_SHAPE;
+        if (!bs_aligned(a.packed[j], 16) || !bs_aligned(a.vt[j], 16) || !bs_aligned(a.u[j], 8)) return BS_ERR_SHAPE;
+        ldy += a.M[j];
+    }
+    if (mode == EPI_SWIGLU) {
+        if (a.n != 2 || a.M[0] != a.M[1]) return BS_ERR_SHAPE;
+        ldy = a.M[0];
+    }
+    const int tp = pass_tokens(T);
+    const Plan p = make_plan(a.I, a.M, a.n, N, tp);
+    if (!workspace || workspace_bytes < p.part_total * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
+    float *part = (float *)workspace;
+    GemvGroup g;
+    RedGroup r;
+    g.n = r.n = a.n;
+    r.mode = mode;
+    int y_off = 0, blocks = 0;
+    for (int j = 0; j < a.n; j++) {
+        g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
+                         p.first_wg[j], p.sp[j]};
+        r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks, p.sp[j]};
+        y_off += a.M[j];
+        if (mode != EPI_SWIGLU || j == 0) blocks += tp * (int)bs_cdiv(a.M[j], RED_OUT);
+    }
+    for (int j = a.n; j < GEMV_MAX_GROUP; j++) { g.m[j] = g.m[0]; r.m[j] = r.m[0]; }
+    for (int t0 = 0; t0 < T; t0 += tp) {
+        const int tn = (T - t0 < tp) ? T - t0 : tp;
+        const half_t *xp = x + (int64_t)t0 * N;
+        int st;
+        switch (tn) {
+            case 1: st = launch_T<1>(p, g, xp, N, K, s); break;
+            case 2: st = launch_T<2>(p, g, xp, N, K, s); break;
+            case 3: st = launch_T<3>(p, g, xp, N, K, s); break;
+            default: st = launch_T<4>(p, g, xp, N, K, s); break;
+        }
+        if (st != BS_OK) return st;
+        // the partial areas are laid out for tp tokens; a shorter last pass uses its own stride
+        RedGroup rr = r;
+        int nblocks = blocks;
+        if (tn != tp) {
+            nblocks = 0;
+            for (int j = 0; j < a.n; j++) {
+                rr.m[j].first_block = nblocks;
+                if (mode != EPI_SWIGLU || j == 0) nblocks += tn * (int)bs_cdiv(a.M[j], RED_OUT);
+            }
+        }
+        gemv_reduce_kernel<<<nblocks, RED_OUT * RED_SL, 0, s>>>(rr, residual ? residual + (int64_t)t0 * ldy : nullptr,
+                                                                y + (int64_t)t0 * ldy, tn, ldy,
+                                                                p.waves * p.R * 16, p.n_chunks);
+        BS_LAUNCH_CHECK();
+    }
+    return BS_OK;
 }
 
 }  // namespace
 
-static bool gemv_shape_ok(int I, int M, int N, int T) {
-    // per-block byte offsets are kept in 32 bits inside the kernel
-    return I >= 1 && T >= 1 && T <= 8 && N % CH == 0 && M >= 1 && (int64_t)M * N < ((int64_t)1 << 31);
-}
-
-// Tokens are processed in passes of at most four (LDS holds Z for four tokens).
-static int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
-
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T) {
     (void)K;
     if (!gemv_shape_ok(I, M, N, T)) return 0;
-    Plan p = make_plan(I, M, N, pass_tokens(T));
-    return (int64_t)I * p.kmax * pass_tokens(T) * M * (int64_t)sizeof(float);
+    const Plan p = make_plan(&I, &M, 1, N, pass_tokens(T));
+    return p.part_total * (int64_t)sizeof(float);
+}
+
+int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, int K, int T) {
+    (void)K;
+    if (n < 1 || n > GEMV_MAX_GROUP) return 0;
+    for (int j = 0; j < n; j++)
+        if (!gemv_shape_ok(I[j], M[j], N, T)) return 0;
+    const Plan p = make_plan(I, M, n, N, pass_tokens(T));
+    return p.part_total * (int64_t)sizeof(float);
 }
 
 // Which instantiation and grid a decode forward of these dimensions runs
@@ -494,11 +668,11 @@ int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T) {
 void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax) {
     *waves = *row_tiles_per_wave = *grid = *kmax = 0;
     if (!gemv_shape_ok(I, M, N, T)) return;
-    const Plan p = make_plan(I, M, N, pass_tokens(T));
+    const Plan p = make_plan(&I, &M, 1, N, pass_tokens(T));
     *waves = p.waves;
     *row_tiles_per_wave = p.R;
     *grid = p.grid;
-    *kmax = p.kmax;
+    *kmax = p.kmax[0];
 }
 
 // Returns BS_ERR_SHAPE when the fast path does not apply (the caller falls
@@ -506,29 +680,23 @@ void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_pe
 int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
                    const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
                    void *workspace, int64_t workspace_bytes, hipStream_t s) {
-    if (!gemv_shape_ok(I, M, N, T)) return BS_ERR_SHAPE;
-    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 8)) return BS_ERR_SHAPE;
-    const int64_t need = bs_gemv_workspace_bytes(I, M, N, K, T);
-    if (!workspace || workspace_bytes < need) return BS_ERR_WORKSPACE;
-    if (I > RED_MAXBLOCKS) return BS_ERR_SHAPE;
-    float *part = (float *)workspace;
-    const int tp = pass_tokens(T);
-    const Plan p = make_plan(I, M, N, tp);
-    for (int t0 = 0; t0 < T; t0 += tp) {
-        const int tn = (T - t0 < tp) ? T - t0 : tp;
-        const half_t *xp = x + (int64_t)t0 * N;
-        int st;
-        switch (tn) {
-            case 1: st = launch_T<1>(p, packed, u, vt, xp, part, M, N, K, s); break;
-            case 2: st = launch_T<2>(p, packed, u, vt, xp, part, M, N, K, s); break;
-            case 3: st = launch_T<3>(p, packed, u, vt, xp, part, M, N, K, s); break;
-            default: st = launch_T<4>(p, packed, u, vt, xp, part, M, N, K, s); break;
-        }
-        if (st != BS_OK) return st;
-        gemv_reduce_kernel<<<tn * (int)bs_cdiv(M, RED_OUT), RED_OUT * RED_SL, 0, s>>>(part, bias, y + (int64_t)t0 * M, I, tn, M,
-                                                                   p.waves * p.R * 16, p.row_tiles, p.n_chunks,
-                                                                   p.sp, p.kmax);
-        BS_LAUNCH_CHECK();
+    GroupArgs a;
+    a.n = 1;
+    a.packed[0] = packed; a.u[0] = u; a.vt[0] = vt; a.bias[0] = bias; a.I[0] = I; a.M[0] = M;
+    return launch_group(a, N, K, x, T, EPI_NONE, nullptr, y, workspace, workspace_bytes, s);
+}
+
+int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
+                         const half_t *const *bias, const int *I, const int *M, int N, int K, const half_t *x, int T,
+                         int mode, const half_t *residual, half_t *y, void *workspace, int64_t workspace_bytes,
+                         hipStream_t s) {
+    if (n < 1 || n > GEMV_MAX_GROUP) return BS_ERR_SHAPE;
+    if (mode == EPI_RESIDUAL && !residual) return BS_ERR_NULL;
+    GroupArgs a;
+    a.n = n;
+    for (int j = 0; j < n; j++) {
+        a.packed[j] = packed[j]; a.u[j] = u[j]; a.vt[j] = vt[j]; a.bias[j] = bias ? bias[j] : nullptr;
+        a.I[j] = I[j]; a.M[j] = M[j];
     }
-    return BS_OK;
+    return launch_group(a, N, K, x, T, mode, residual, y, workspace, workspace_bytes, s);
 }

@@ -81,6 +81,116 @@ def bitstack_forward_hip(packed_sign, u, vt, x, bias=None):
     return y.view(x.shape[:-1] + (M,))
 
 
+class MatrixGroup:
+    """Up to four stacked BitStack matrices with the same in_features and rank that
+    are always applied to the same input (q/k/v, gate/up): the argument block of
+    bs_forward_group, built once.  Keeps the tensors alive."""
+
+    def __init__(self, mats):
+        # mats: sequence of (packed_sign [I, M*N/8], u [I, M, K], vt [I, K, N], bias or None)
+        self.tensors = []
+        self.M = []
+        arr = (_lib.bs_matrix * len(mats))()
+        N = K = None
+        for j, (q, u, vt, bias) in enumerate(mats):
+            _lib.require_gpu(q, u, vt, bias)
+            I, M, n, k = _dims(u, vt)
+            if N is None:
+                N, K = n, k
+            elif (n, k) != (N, K):
+                raise ValueError("matrices of a group share in_features and rank")
+            if q.dtype != torch.uint8 or q.numel() != I * ((M * n + 7) // 8):
+                raise ValueError("packed signs do not match u / vt")
+            q, u, vt = q.contiguous(), _f16c(u), _f16c(vt)
+            bias = None if bias is None else _f16c(bias)
+            self.tensors.append((q, u, vt, bias))
+            arr[j].packed, arr[j].u, arr[j].vt = q.data_ptr(), u.data_ptr(), vt.data_ptr()
+            arr[j].bias = None if bias is None else bias.data_ptr()
+            arr[j].I, arr[j].M = I, M
+            self.M.append(M)
+        self.arr, self.n, self.N, self.K = arr, len(mats), N, K
+        self.dev = mats[0][0].device
+        self._need = {}
+
+    @classmethod
+    def from_modules(cls, modules):
+        """modules: BitStackLinear objects after stack_blocks(), using their first w_bit blocks."""
+        mats = []
+        for m in modules:
+            q, u, vt = m._stacked()
+            mats.append((q, u, vt, m.bias))
+        return cls(mats)
+
+    def workspace_bytes(self, T):
+        if T not in self._need:
+            self._need[T] = int(_lib.lib().bs_forward_group_workspace_bytes(self.arr, self.n, self.N, self.K, T))
+        return self._need[T]
+
+
+def bitstack_forward_group_hip(group: MatrixGroup, x, epilogue=_lib.EPI_NONE, residual=None, out=None):
+    """All matrices of `group` applied to x [T, N] (T <= 8) in one launch pair, with
+    the outputs side by side [T, sum M] (EPI_NONE), plus `residual` (EPI_RESIDUAL),
+    or silu(first) * second [T, M] (EPI_SWIGLU).  What three (two) module calls and
+    the element-wise ops after them do in a decoder layer."""
+    dev = _lib.require_gpu(x, residual, out)
+    x2 = _f16c(x).view(-1, group.N)
+    T = x2.shape[0]
+    width = group.M[0] if epilogue == _lib.EPI_SWIGLU else sum(group.M)
+    need = group.workspace_bytes(T)
+    if need < 0:
+        _lib.check(need, "bs_forward_group_workspace_bytes")
+    if residual is not None:
+        residual = _f16c(residual)
+        if residual.numel() != T * width:
+            raise ValueError("residual does not match the output")
+    y = out if out is not None else torch.empty((T, width), dtype=torch.float16, device=dev)
+    if y.dtype != torch.float16 or not y.is_contiguous() or y.numel() != T * width:
+        raise ValueError("out must be a contiguous fp16 [T, width] tensor")
+    ws = _lib.workspace(dev, need)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().bs_forward_group(group.arr, group.n, group.N, group.K, _lib.ptr(x2), T, epilogue,
+                                               _lib.ptr(residual), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                                               _lib.stream_ptr(dev)), "bs_forward_group")
+    return y
+
+
+def rmsnorm_hip(x, weight, eps, out=None):
+    """weight * fp16(x * rsqrt(mean(x^2) + eps)) over the last dimension."""
+    dev = _lib.require_gpu(x, weight, out)
+    H = x.shape[-1]
+    x2, weight = _f16c(x).view(-1, H), _f16c(weight)
+    y = out if out is not None else torch.empty_like(x2)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().bs_rmsnorm_f16(_lib.ptr(x2), _lib.ptr(weight), _lib.ptr(y), x2.shape[0], H, float(eps),
+                                             _lib.stream_ptr(dev)), "bs_rmsnorm_f16")
+    return y.view(x.shape)
+
+
+def attention_decode_hip(qkv, kcache, vcache, cos, sin, pos, heads, kv_heads, out=None):
+    """One decode position for B sequences: RoPE on q and k of qkv [B, (heads + 2 kv) * d],
+    append k, v at *pos to the caches [B, kv, max_len, d], attention over 0..*pos;
+    returns [B, heads * d].  `pos` is a one-element int64 device tensor."""
+    dev = _lib.require_gpu(qkv, kcache, vcache, cos, sin, pos, out)
+    B = qkv.shape[0]
+    d = kcache.shape[-1]
+    max_len = kcache.shape[-2]
+    if qkv.dtype != torch.float16 or not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * d:
+        raise ValueError("qkv must be contiguous fp16 [B, (heads + 2 kv_heads) * head_dim]")
+    for c in (kcache, vcache):
+        if c.dtype != torch.float16 or not c.is_contiguous() or c.numel() != B * kv_heads * max_len * d:
+            raise ValueError("caches must be contiguous fp16 [B, kv_heads, max_len, head_dim]")
+    if pos.dtype != torch.int64 or pos.numel() != 1:
+        raise ValueError("pos must be a one-element int64 tensor")
+    if cos.shape != (max_len, d // 2) or sin.shape != (max_len, d // 2) or not cos.is_contiguous() or not sin.is_contiguous():
+        raise ValueError("cos / sin must be contiguous [max_len, head_dim / 2]")
+    y = out if out is not None else torch.empty((B, heads * d), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().bs_attention_decode_f16(_lib.ptr(qkv), _lib.ptr(kcache), _lib.ptr(vcache), _lib.ptr(_f16c(cos)),
+                                                      _lib.ptr(_f16c(sin)), _lib.ptr(pos), _lib.ptr(y), B, heads, kv_heads,
+                                                      d, max_len, _lib.stream_ptr(dev)), "bs_attention_decode_f16")
+    return y
+
+
 def linear_f16_hip(x, w, bias=None):
     """F.linear on the library's own MFMA kernel (fp16 in, fp32 accumulate)."""
     dev = _lib.require_gpu(x, w, bias)

@@ -7,10 +7,10 @@ reference's format, {"layer.{L}.self_attn.q_proj": n_blocks, ...}
 (bitstack/utils/decompose.py:14, bitstack/utils/model_utils.py:53-66); embed_tokens
 and lm_head stay dense fp16, as in the reference (only the decoder layers are
 walked, bitstack/utils/scale_utils.py:212-221).  Everything around the linears
-(RMSNorm, RoPE, attention over a static KV cache, SiLU gate) is plain torch: the
-subject of the measurement is the linear path.  One decode step has static shapes
-and reads its position from a device tensor, so it can be captured in a HIP graph
-and replayed.
+(RMSNorm, RoPE, attention over a static KV cache, SiLU gate) is plain torch in
+step() and the library's decode-step kernels in step_fused().  One decode step has
+static shapes and reads its position from a device tensor, so it can be captured in
+a HIP graph and replayed.
 """
 from __future__ import annotations
 
@@ -20,7 +20,10 @@ from dataclasses import dataclass
 import torch
 import torch.nn.functional as F
 
+from bitstack_amd._lib import EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU
 from bitstack_amd.modules.BitStackLinear import BitStackLinear
+from bitstack_amd.utils.inference_utils import (MatrixGroup, attention_decode_hip, bitstack_forward_group_hip,
+                                                rmsnorm_hip)
 
 PROJ = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
         "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")
@@ -98,10 +101,18 @@ def _synthetic_bitstack(m, n, blocks, k, dev, gen, name):
 
 
 class SyntheticLlamaDecoder:
-    """Batch-1 greedy decode with a static KV cache of `max_len` positions."""
+    """Greedy decode of `batch` sequences in lock step (all at the same position)
+    with a static KV cache of `max_len` positions.
 
-    def __init__(self, shape: LlamaShape, config: dict, max_len: int, device, seed=0):
-        self.s, self.dev, self.max_len = shape, torch.device(device), max_len
+    step()        every op around the linears is a torch op, one BitStackLinear
+                  call per projection (the structure the reference runs);
+    step_fused()  four launch pairs per layer for the seven linears (q/k/v in one,
+                  o with the residual add, gate/up with the SiLU product, down with
+                  the residual add), one RMSNorm and one attention kernel between
+                  them, all from the library."""
+
+    def __init__(self, shape: LlamaShape, config: dict, max_len: int, device, seed=0, batch=1):
+        self.s, self.dev, self.max_len, self.batch = shape, torch.device(device), max_len, batch
         g = torch.Generator(device=self.dev).manual_seed(seed)
         h = shape.hidden
         self.embed = (torch.randn(shape.vocab, h, device=self.dev, generator=g) * 0.02).half()
@@ -116,14 +127,16 @@ class SyntheticLlamaDecoder:
                 row[p] = _synthetic_bitstack(m, n, config[f"layer.{L}.{p}"], shape.k, self.dev, g, f"layer.{L}.{p}")
             self.lin.append(row)
         d = shape.head_dim
-        self.kcache = torch.zeros(shape.layers, shape.kv_heads, max_len, d, device=self.dev, dtype=torch.float16)
+        self.kcache = torch.zeros(shape.layers, batch, shape.kv_heads, max_len, d, device=self.dev, dtype=torch.float16)
         self.vcache = torch.zeros_like(self.kcache)
         inv = 1.0 / (shape.rope_theta ** (torch.arange(0, d, 2, device=self.dev, dtype=torch.float32) / d))
         ang = torch.arange(max_len, device=self.dev, dtype=torch.float32)[:, None] * inv[None, :]
-        self.cos, self.sin = ang.cos().half(), ang.sin().half()            # [max_len, d/2]
+        self.cos, self.sin = ang.cos().half().contiguous(), ang.sin().half().contiguous()   # [max_len, d/2]
         self.pos = torch.zeros(1, device=self.dev, dtype=torch.long)       # next position to write
-        self.token = torch.zeros(1, device=self.dev, dtype=torch.long)
+        self.token = torch.zeros(batch, device=self.dev, dtype=torch.long)
         self.span = torch.arange(max_len, device=self.dev)
+        self.logits = None
+        self._groups = None
 
     def weight_bytes(self):
         b = self.embed.numel() * 2 + self.lm_head.numel() * 2
@@ -132,11 +145,16 @@ class SyntheticLlamaDecoder:
                 b += m.qweight.numel() + 2 * (m.u.numel() + m.vt.numel())
         return b
 
+    def reset(self):
+        self.pos.zero_()
+        self.kcache.zero_()
+        self.vcache.zero_()
+
     def _rms(self, x, w):
         v = x.float()
         return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.s.rms_eps)).half() * w
 
-    def _rope(self, x, cos, sin):          # x [heads, d], rotate-half convention
+    def _rope(self, x, cos, sin):          # x [..., d], rotate-half convention
         d2 = x.shape[-1] // 2
         a, b = x[..., :d2], x[..., d2:]
         return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
@@ -144,37 +162,81 @@ class SyntheticLlamaDecoder:
     @torch.no_grad()
     def step(self):
         """Consume self.token at self.pos, write the greedy next token, advance."""
-        s = self.s
-        x = self.embed.index_select(0, self.token)                       # [1, h]
+        s, B = self.s, self.batch
+        x = self.embed.index_select(0, self.token)                       # [B, h]
         cos = self.cos.index_select(0, self.pos)
         sin = self.sin.index_select(0, self.pos)
-        mask = (self.span <= self.pos).view(1, 1, self.max_len)
+        mask = (self.span <= self.pos).view(1, 1, 1, self.max_len)
+        rep = s.heads // s.kv_heads
         for L in range(s.layers):
             lin = self.lin[L]
             hn = self._rms(x, self.norm_w[L, 0])
-            q = lin["self_attn.q_proj"](hn).view(s.heads, s.head_dim)
-            k = lin["self_attn.k_proj"](hn).view(s.kv_heads, s.head_dim)
-            v = lin["self_attn.v_proj"](hn).view(s.kv_heads, s.head_dim)
+            q = lin["self_attn.q_proj"](hn).view(B, s.heads, s.head_dim)
+            k = lin["self_attn.k_proj"](hn).view(B, s.kv_heads, s.head_dim)
+            v = lin["self_attn.v_proj"](hn).view(B, s.kv_heads, s.head_dim)
             q, k = self._rope(q, cos, sin), self._rope(k, cos, sin)
-            self.kcache[L].index_copy_(1, self.pos, k.unsqueeze(1))
-            self.vcache[L].index_copy_(1, self.pos, v.unsqueeze(1))
-            rep = s.heads // s.kv_heads
-            qg = q.view(s.kv_heads, rep, s.head_dim)
-            att = torch.matmul(qg, self.kcache[L].transpose(1, 2)) / math.sqrt(s.head_dim)   # [kv, rep, max_len]
+            self.kcache[L].index_copy_(2, self.pos, k.unsqueeze(2))
+            self.vcache[L].index_copy_(2, self.pos, v.unsqueeze(2))
+            qg = q.view(B, s.kv_heads, rep, s.head_dim)
+            att = torch.matmul(qg, self.kcache[L].transpose(2, 3)) / math.sqrt(s.head_dim)   # [B, kv, rep, max_len]
             att = att.masked_fill(~mask, float("-inf")).float().softmax(-1).half()
-            ctx = torch.matmul(att, self.vcache[L]).reshape(1, s.hidden)
+            ctx = torch.matmul(att, self.vcache[L]).reshape(B, s.hidden)
             x = x + lin["self_attn.o_proj"](ctx)
             hn = self._rms(x, self.norm_w[L, 1])
             gate = lin["mlp.gate_proj"](hn)
             up = lin["mlp.up_proj"](hn)
             x = x + lin["mlp.down_proj"](F.silu(gate) * up)
-        logits = F.linear(self._rms(x, self.final_norm), self.lm_head)
-        self.token.copy_(logits.argmax(-1))
+        self.logits = F.linear(self._rms(x, self.final_norm), self.lm_head)
+        self.token.copy_(self.logits.argmax(-1))
         self.pos.add_(1)
 
-    def prefill_positions(self, prompt: torch.Tensor):
-        """Feed a prompt token by token (the measurement is about decode)."""
+    def _build_groups(self):
+        s, B = self.s, self.batch
+        self._groups = []
+        for L in range(s.layers):
+            lin = self.lin[L]
+            self._groups.append({
+                "qkv": MatrixGroup.from_modules([lin["self_attn.q_proj"], lin["self_attn.k_proj"], lin["self_attn.v_proj"]]),
+                "o": MatrixGroup.from_modules([lin["self_attn.o_proj"]]),
+                "gate_up": MatrixGroup.from_modules([lin["mlp.gate_proj"], lin["mlp.up_proj"]]),
+                "down": MatrixGroup.from_modules([lin["mlp.down_proj"]]),
+            })
+        f16 = dict(dtype=torch.float16, device=self.dev)
+        self._hn = torch.empty(B, s.hidden, **f16)
+        self._qkv = torch.empty(B, (s.heads + 2 * s.kv_heads) * s.head_dim, **f16)
+        self._ctx = torch.empty(B, s.hidden, **f16)
+        self._act = torch.empty(B, s.intermediate, **f16)
+        self._xa = torch.empty(B, s.hidden, **f16)
+        self._xb = torch.empty(B, s.hidden, **f16)
+
+    @torch.no_grad()
+    def step_fused(self):
+        """Same step on the library's grouped forwards and decode-step kernels."""
+        if self._groups is None:
+            self._build_groups()
+        s = self.s
+        xa, xb = self._xa, self._xb
+        torch.index_select(self.embed, 0, self.token, out=xa)
+        for L in range(s.layers):
+            grp = self._groups[L]
+            rmsnorm_hip(xa, self.norm_w[L, 0], s.rms_eps, out=self._hn)
+            bitstack_forward_group_hip(grp["qkv"], self._hn, EPI_NONE, out=self._qkv)
+            attention_decode_hip(self._qkv, self.kcache[L], self.vcache[L], self.cos, self.sin, self.pos,
+                                 s.heads, s.kv_heads, out=self._ctx)
+            bitstack_forward_group_hip(grp["o"], self._ctx, EPI_RESIDUAL, residual=xa, out=xb)
+            rmsnorm_hip(xb, self.norm_w[L, 1], s.rms_eps, out=self._hn)
+            bitstack_forward_group_hip(grp["gate_up"], self._hn, EPI_SWIGLU, out=self._act)
+            bitstack_forward_group_hip(grp["down"], self._act, EPI_RESIDUAL, residual=xb, out=xa)
+        rmsnorm_hip(xa, self.final_norm, s.rms_eps, out=self._hn)
+        self.logits = F.linear(self._hn, self.lm_head)
+        self.token.copy_(self.logits.argmax(-1))
+        self.pos.add_(1)
+
+    def prefill_positions(self, prompt: torch.Tensor, fused=False):
+        """Feed a prompt token by token (the measurement is about decode).  `prompt`
+        is [len] (the same for every sequence) or [batch, len]."""
         self.pos.zero_()
-        for tkn in prompt.tolist():
-            self.token.fill_(tkn)
-            self.step()
+        prompt = prompt.view(1, -1).expand(self.batch, -1) if prompt.dim() == 1 else prompt
+        for j in range(prompt.shape[1]):
+            self.token.copy_(prompt[:, j])
+            (self.step_fused if fused else self.step)()

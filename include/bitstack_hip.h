@@ -125,6 +125,68 @@ int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles
 int bs_linear_f16(const void *x, const void *w, const void *bias, void *y,
                   int T, int M, int N, void *stream);
 
+/*
+ * ---- decode step: several matrices per launch, fused epilogues -----------
+ * One decode forward (T <= 8 tokens) of up to 4 compressed matrices that read
+ * the same x, in one kernel pair: what q_proj/k_proj/v_proj (or gate_proj/
+ * up_proj) of a decoder layer do with three (two) BitStackLinear.forward calls,
+ * bitstack/modules/BitStackLinear.py:88-157, each as in bs_forward.  All share
+ * N and K; block counts and row counts are per matrix.
+ *   BS_EPI_NONE      y[T, sum M_j]: the outputs side by side, matrix j at column
+ *                    offset M_0 + ... + M_{j-1}
+ *   BS_EPI_RESIDUAL  the same, plus residual[T, sum M_j] (fp16 add of the fp16
+ *                    result, as `x + proj(h)` in the decoder layer)
+ *   BS_EPI_SWIGLU    n == 2, M_0 == M_1: y[T, M_0] = silu(first) * second
+ *                    computed from the fp16-rounded results, as
+ *                    `act_fn(gate_proj(h)) * up_proj(h)` in the MLP
+ * Only shapes the decode kernel takes (every matrix: N % 512 == 0,
+ * M * N < 2^31, alignment as bs_forward); anything else returns BS_ERR_SHAPE
+ * and the caller issues bs_forward per matrix.  Workspace as bs_forward, size
+ * from bs_forward_group_workspace_bytes (negative = status).
+ */
+#define BS_EPI_NONE      0
+#define BS_EPI_RESIDUAL  1
+#define BS_EPI_SWIGLU    2
+#define BS_MAX_GROUP     4
+
+typedef struct bs_matrix {
+    const uint8_t *packed;   /* [I, M*N/8] */
+    const void *u;           /* f16 [I, M, K] */
+    const void *vt;          /* f16 [I, K, N] */
+    const void *bias;        /* f16 [M] or NULL */
+    int32_t I, M;
+} bs_matrix;
+
+int64_t bs_forward_group_workspace_bytes(const bs_matrix *mats, int n, int N, int K, int T);
+
+int bs_forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, int T,
+                     int epilogue, const void *residual, void *y,
+                     void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * y[T, H] = weight o fp16( x * rsqrt(mean(x^2) + eps) ), statistics in fp32:
+ * the RMSNorm in front of the attention and MLP linears of a decoder layer
+ * (the reference leaves it to the Hugging Face model it patches,
+ * bitstack/utils/scale_utils.py:212-221 walks `model.model.layers`).
+ * H % 8 == 0, H <= 16384, 16-byte aligned rows.
+ */
+int bs_rmsnorm_f16(const void *x, const void *weight, void *y, int T, int H, float eps, void *stream);
+
+/*
+ * One decode position of grouped-query attention for B sequences that are all
+ * at position *pos (device int64): rotate q and k of `qkv`
+ * [B, (heads + 2 kv_heads) * head_dim] (rotate-half RoPE with cos/sin
+ * [max_len, head_dim / 2]), store k and v at *pos in the caches
+ * [B, kv_heads, max_len, head_dim], softmax(q k^T / sqrt(head_dim)) v over
+ * positions 0..*pos, write out[B, heads * head_dim].  head_dim == 128,
+ * max_len <= 8192.  The step between the q/k/v and o linears of a decoder
+ * layer; no counterpart inside the reference repository (Hugging Face's
+ * LlamaAttention).
+ */
+int bs_attention_decode_f16(const void *qkv, void *kcache, void *vcache, const void *cos, const void *sin,
+                            const int64_t *pos, void *out, int B, int heads, int kv_heads, int head_dim,
+                            int max_len, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,233 @@
+"""The decode step around the compressed linears on a real MI355X, through the C ABI:
+grouped forwards (several matrices per launch, fused epilogues) against the C oracle,
+RMSNorm and the rotary attention step against fp64 restatements (oracle/llama_oracle.py,
+itself pinned against `transformers`), and the whole fused step against the torch-op step
+and against the float64 decoder on the rebuilt dense weights.  Tolerances as for the
+layer outputs: max|d|/max|ref| <= 1e-2, mean|d|/mean|ref| <= 1e-3 unless stated."""
+import numpy as np
+import pytest
+import torch
+
+from bitstack_amd import _lib
+from bitstack_amd.utils import inference_utils as IU
+from bitstack_amd.utils.llama_decode import LlamaShape, PROJ, SyntheticLlamaDecoder
+from bitstack_amd.utils.synthetic import synthetic_layer
+from oracle import bitstack_oracle as O
+from oracle import c_oracle as C
+from oracle import llama_oracle as LO
+
+pytestmark = pytest.mark.gpu
+MAX_REL, MEAN_REL = 1e-2, 1e-3
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def assert_close(got, ref, what, max_rel=MAX_REL, mean_rel=MEAN_REL):
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    d = np.abs(got - ref)
+    mx, mn = d.max() / max(np.abs(ref).max(), 1e-30), d.mean() / max(np.abs(ref).mean(), 1e-30)
+    print(f"{what}: max_rel={mx:.3e} mean_rel={mn:.3e}", flush=True)
+    assert mx <= max_rel and mn <= mean_rel, f"{what}: max_rel={mx:.3e} mean_rel={mn:.3e}"
+
+
+def make_group(shapes, N, T, seed, bias=False):
+    """shapes: [(I, M)]; returns (MatrixGroup on the GPU, x on the CPU, fp64 reference outputs per matrix)."""
+    mats, refs, x = [], [], None
+    for j, (I, M) in enumerate(shapes):
+        q, u, vt, xj = synthetic_layer(M, N, I, T, seed=seed + j, signed_factors=True)
+        x = xj if x is None else x
+        b = torch.randn(M, generator=torch.Generator().manual_seed(seed + 50 + j)).half() * 0.05 if bias else None
+        refs.append(C.forward_f64(q.numpy(), u.numpy(), vt.numpy(), x.numpy(), None if b is None else b.numpy()))
+        mats.append((q.to(dev()), u.to(dev()), vt.to(dev()), None if b is None else b.to(dev())))
+    return IU.MatrixGroup(mats), x, refs
+
+
+GROUP_CASES = [([(3, 512), (5, 128), (2, 128)], 512, 1), ([(3, 4096), (5, 1024), (2, 1024)], 4096, 1),
+               ([(2, 1024), (4, 256)], 1024, 2), ([(1, 300), (2, 77), (3, 64), (1, 512)], 1536, 3),
+               ([(2, 512), (3, 256)], 1024, 4), ([(2, 512), (1, 256)], 512, 5), ([(2, 256), (2, 256)], 1024, 8)]
+
+
+@pytest.mark.parametrize("shapes,N,T", GROUP_CASES)
+def test_group_forward_side_by_side(shapes, N, T):
+    print(f"group forward {shapes} N={N} T={T}", flush=True)
+    grp, x, refs = make_group(shapes, N, T, seed=11, bias=(T % 2 == 0))
+    y = IU.bitstack_forward_group_hip(grp, x.to(dev())).cpu().numpy()
+    assert y.shape == (T, sum(m for _, m in shapes)) and y.dtype == np.float16
+    assert_close(y, np.concatenate(refs, axis=1), "group vs fp64")
+    # and the same numbers as one bs_forward per matrix, up to the order of the fp32 partial sums
+    off = 0
+    for (q, u, vt, b), (_, M) in zip(grp.tensors, shapes):
+        single = IU.bitstack_forward_hip(q, u, vt, x.to(dev()), b).cpu().numpy()
+        assert_close(y[:, off:off + M], single, "group vs single", 2e-3, 2e-4)
+        off += M
+
+
+@pytest.mark.parametrize("I,M,N,T", [(3, 512, 1024, 1), (2, 4096, 4096, 1), (2, 256, 512, 6)])
+def test_group_forward_residual(I, M, N, T):
+    print(f"group residual I={I} M={M} N={N} T={T}", flush=True)
+    grp, x, refs = make_group([(I, M)], N, T, seed=21)
+    res = (torch.randn(T, M, generator=torch.Generator().manual_seed(2)) * 0.1).half()
+    y = IU.bitstack_forward_group_hip(grp, x.to(dev()), _lib.EPI_RESIDUAL, residual=res.to(dev())).cpu().numpy()
+    assert_close(y, refs[0] + res.double().numpy(), "residual vs fp64")
+    plain = IU.bitstack_forward_group_hip(grp, x.to(dev())).cpu()
+    assert np.array_equal(y, (res.float() + plain.float()).half().numpy())        # exactly the fp16 add of the fp16 result
+
+
+@pytest.mark.parametrize("I0,I1,M,N,T", [(3, 2, 1024, 512, 1), (2, 4, 14336, 4096, 1), (2, 2, 512, 1024, 7)])
+def test_group_forward_swiglu(I0, I1, M, N, T):
+    print(f"group swiglu I={I0},{I1} M={M} N={N} T={T}", flush=True)
+    grp, x, refs = make_group([(I0, M), (I1, M)], N, T, seed=31)
+    # scale so that the gate spans the non-linear range of silu
+    y = IU.bitstack_forward_group_hip(grp, x.to(dev()), _lib.EPI_SWIGLU).cpu().numpy()
+    assert y.shape == (T, M)
+    assert_close(y, LO.silu(refs[0]) * refs[1], "swiglu vs fp64", 2e-2, 2e-3)
+    both = IU.bitstack_forward_group_hip(grp, x.to(dev())).cpu()
+    gate, up = both[:, :M], both[:, M:]
+    want = (torch.nn.functional.silu(gate.float()).half().float() * up.float()).half().numpy()
+    d = np.abs(y.astype(np.float64) - want.astype(np.float64))
+    assert d.max() <= 2e-3 * max(np.abs(want).max(), 1e-30)       # same rounding points; expf differs in the last bit at most
+
+
+def test_group_rejects_what_the_decode_kernel_does_not_take():
+    grp, x, _ = make_group([(1, 64), (1, 64)], 512, 1, seed=1)
+    with pytest.raises(RuntimeError):
+        IU.bitstack_forward_group_hip(grp, torch.zeros(9, 512, dtype=torch.float16, device=dev()))    # more than 8 tokens
+    grp2, _, _ = make_group([(1, 64), (1, 128)], 512, 1, seed=1)
+    with pytest.raises(RuntimeError):
+        IU.bitstack_forward_group_hip(grp2, x.to(dev()), _lib.EPI_SWIGLU)                               # unequal M
+    with pytest.raises(RuntimeError):
+        IU.bitstack_forward_group_hip(grp, x.to(dev()), _lib.EPI_RESIDUAL)                               # no residual
+
+
+@pytest.mark.parametrize("T,H", [(1, 4096), (3, 512), (8, 8192), (2, 16384), (5, 264)])
+def test_rmsnorm(T, H):
+    print(f"rmsnorm T={T} H={H}", flush=True)
+    g = torch.Generator().manual_seed(H + T)
+    x = (torch.randn(T, H, generator=g) * 3).half()
+    w = (1 + 0.3 * torch.randn(H, generator=g)).half()
+    y = IU.rmsnorm_hip(x.to(dev()), w.to(dev()), 1e-5).cpu()
+    assert_close(y.numpy(), LO.rmsnorm(x.double().numpy(), w.double().numpy(), 1e-5), "rmsnorm vs fp64", 2e-3, 5e-4)
+    # the rounding points of the usual implementation: normalised value to fp16, then times the weight
+    v = x.float()
+    want = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
+    assert (y.float() - want.float()).abs().max() <= 2 * torch.finfo(torch.float16).eps * want.float().abs().max()
+
+
+@pytest.mark.parametrize("B,heads,kv", [(1, 32, 8), (3, 4, 2), (2, 8, 8)])
+def test_attention_decode_steps(B, heads, kv):
+    print(f"attention B={B} heads={heads} kv={kv}", flush=True)
+    d, max_len, steps = 128, 40, 37
+    g = torch.Generator().manual_seed(heads)
+    cos64, sin64 = LO.rope_tables(max_len, d, 500000.0)
+    cos, sin = torch.from_numpy(cos64).half(), torch.from_numpy(sin64).half()
+    kc = torch.zeros(B, kv, max_len, d, dtype=torch.float16, device=dev())
+    vc = torch.zeros_like(kc)
+    pos = torch.zeros(1, dtype=torch.long, device=dev())
+    kref = np.zeros((B, kv, max_len, d))
+    vref = np.zeros((B, kv, max_len, d))
+    for p in range(steps):
+        qkv = torch.randn(B, (heads + 2 * kv) * d, generator=g).half()
+        out = IU.attention_decode_hip(qkv.to(dev()), kc, vc, cos.to(dev()), sin.to(dev()), pos, heads, kv).cpu().numpy()
+        pos.add_(1)
+        x = qkv.double().numpy()
+        c, s = cos[p].double().numpy(), sin[p].double().numpy()
+        for b in range(B):
+            q = LO.rope(x[b, :heads * d].reshape(heads, d), c, s)
+            kref[b, :, p] = LO.rope(x[b, heads * d:(heads + kv) * d].reshape(kv, d), c, s)
+            vref[b, :, p] = x[b, (heads + kv) * d:].reshape(kv, d)
+            # the kernel attends over the fp16 cache it wrote; follow that for the reference of later steps
+            want = LO.attention_decode(q, kref[b], vref[b], p + 1).reshape(-1)
+            if p in (0, 1, 15, 16, 17, steps - 1):
+                assert_close(out[b], want, f"attention step {p} seq {b}", 1e-2, 2e-3)
+    assert_close(kc.cpu().numpy()[:, :, :steps], kref[:, :, :steps], "k cache", 2e-3, 5e-4)
+    assert np.array_equal(vc.cpu().numpy()[:, :, :steps], vref[:, :, :steps].astype(np.float16))
+    assert float(kc[:, :, steps:].abs().max()) == 0.0 and float(vc[:, :, steps:].abs().max()) == 0.0
+
+
+def test_attention_position_outside_the_cache_writes_zeros_and_touches_nothing():
+    kc = torch.zeros(1, 2, 8, 128, dtype=torch.float16, device=dev())
+    vc = torch.zeros_like(kc)
+    tab = torch.ones(8, 64, dtype=torch.float16, device=dev())
+    qkv = torch.ones(1, 8 * 128, dtype=torch.float16, device=dev())
+    out = IU.attention_decode_hip(qkv, kc, vc, tab, tab, torch.tensor([8], device=dev()), 4, 2)
+    assert float(out.abs().max()) == 0.0 and float(kc.abs().max()) == 0.0
+
+
+SMALL = LlamaShape(layers=2, hidden=512, intermediate=1024, heads=4, kv_heads=2, vocab=256)
+
+
+def small_config(seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return {f"layer.{L}.{p}": int(torch.randint(1, 5, (1,), generator=g)) for L in range(SMALL.layers) for p in PROJ}
+
+
+def dense_weights(model):
+    """Hugging Face names -> float64 arrays, the compressed linears rebuilt in float64 by the oracle."""
+    w = {"model.embed_tokens.weight": model.embed.double().cpu().numpy(), "lm_head.weight": model.lm_head.double().cpu().numpy(),
+         "model.norm.weight": model.final_norm.double().cpu().numpy()}
+    for L in range(model.s.layers):
+        w[f"model.layers.{L}.input_layernorm.weight"] = model.norm_w[L, 0].double().cpu().numpy()
+        w[f"model.layers.{L}.post_attention_layernorm.weight"] = model.norm_w[L, 1].double().cpu().numpy()
+        for p in PROJ:
+            m = model.lin[L][p]
+            w[f"model.layers.{L}.{p}.weight"] = O.reconstruct_w_exact(m.qweight.cpu().numpy(), m.u.cpu().numpy(), m.vt.cpu().numpy())
+    return w
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_fused_step_matches_torch_step_and_float64_decoder(batch):
+    print(f"fused decode step batch={batch}", flush=True)
+    cfg = small_config()
+    a = SyntheticLlamaDecoder(SMALL, cfg, 24, dev(), seed=4, batch=batch)
+    b = SyntheticLlamaDecoder(SMALL, cfg, 24, dev(), seed=4, batch=batch)
+    # norm weights away from one, factors large enough that the layers matter
+    with torch.no_grad():
+        for m in (a, b):
+            g = torch.Generator(device=dev()).manual_seed(9)
+            m.norm_w.copy_(1 + 0.2 * torch.randn(m.norm_w.shape, device=dev(), generator=g))
+            m.embed.mul_(30.0)
+    w = dense_weights(a)
+    orcs = [LO.LlamaOracle(w, SMALL.layers, SMALL.heads, SMALL.kv_heads, SMALL.head_dim, SMALL.rope_theta, SMALL.rms_eps, 24)
+            for _ in range(batch)]
+    tokens = torch.randint(0, SMALL.vocab, (batch, 10), generator=torch.Generator().manual_seed(1))
+    for j in range(tokens.shape[1]):
+        a.token.copy_(tokens[:, j])
+        b.token.copy_(tokens[:, j])
+        a.step()
+        b.step_fused()
+        la, lb = a.logits.float().cpu().numpy(), b.logits.float().cpu().numpy()
+        assert lb.shape == (batch, SMALL.vocab)
+        for s in range(batch):
+            want = orcs[s].step(int(tokens[s, j]))
+            assert_close(lb[s], want, f"fused vs float64, position {j} seq {s}", 2e-2, 4e-3)
+            assert_close(la[s], want, f"torch step vs float64, position {j} seq {s}", 2e-2, 4e-3)
+    assert int(b.pos) == tokens.shape[1]
+    assert_close(b.kcache.float().cpu().numpy(), a.kcache.float().cpu().numpy(), "k cache fused vs torch", 1e-2, 2e-3)
+
+
+def test_fused_step_replays_in_a_graph():
+    cfg = small_config(1)
+    m = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=2)
+    ref = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=2)
+    m.token.fill_(5)
+    ref.token.fill_(5)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        m.step_fused()                       # warm-up outside capture: workspaces, group argument blocks
+    torch.cuda.current_stream().wait_stream(side)
+    m.reset()
+    m.token.fill_(5)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        m.step_fused()
+    m.reset()
+    m.token.fill_(5)
+    for step in range(6):                    # replays interleaved with eager work, each checked
+        graph.replay()
+        ref.step_fused()
+        torch.cuda.synchronize()
+        assert torch.equal(m.logits, ref.logits), step
+        assert torch.equal(m.token, ref.token) and int(m.pos) == step + 1
