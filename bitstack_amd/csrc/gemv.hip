@@ -350,14 +350,21 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     int rowid = u_begin / n_chunks, c = u_begin % n_chunks;
     set_row(rowid);
     uint4_t cur[R], nxt[R];
+    produce_issue(c);                               // first: Z production only waits for these
     load_signs(cur, c);
-    produce_issue(c);
+    uint32_t warm = 0;
+    {
+        // the flush after the last unit is not preceded by a crossing inside the loop:
+        // pull the u rows it needs towards L2 now (value unused)
+        const int lrow = (u_end - 1) / n_chunks, fi = lrow / row_tiles, frt = lrow % row_tiles;
+        const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
+        warm ^= *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
+    }
     produce_write(0);
     __syncthreads();
 
     // ---- steady state -------------------------------------------------------
     int buf = 0;
-    uint32_t warm = 0;
     for (int unit = u_begin; unit + 1 < u_end; unit++) {
         const bool crossing = c + 1 == n_chunks;    // the next unit starts another row
         const int cn = crossing ? 0 : c + 1;
@@ -393,15 +400,14 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
 
 // y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ) where k
 // runs over the workgroups whose unit range touched (block i, row tile of m), in
-// ascending order.  32 outputs of one row tile per workgroup; the number of
-// partials of every block is worked out once (one thread per block) into LDS,
-// eight threads per output take every eighth block (their loads are independent)
-// and are combined through LDS in a fixed order.
+// ascending order.  32 outputs of one row tile per workgroup; eight threads per
+// output take every eighth block (their loads are independent) and are combined
+// through LDS in a fixed order.
 // Epilogues (applied to the fp16-rounded sums, the way separate fp16 ops would):
 //   EPI_NONE      the matrices' outputs side by side in one row of `ldy` halves
 //   EPI_RESIDUAL  the same plus residual[t, off + m]
 //   EPI_SWIGLU    two matrices of equal M: silu(first) * second, one row of M
-constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;
+constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;   // the last one is a sanity limit on the block count
 
 struct RedMat {
     const float *part;
@@ -414,42 +420,39 @@ struct RedGroup {
     int n, mode;
 };
 
-__device__ __forceinline__ float reduce_partials(const RedMat &r, int T, int t, int m0, int rows_per_tile, int n_chunks,
-                                                 int *nks, float (*red)[RED_OUT]) {
-    const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
-    const int m = m0 + lo;
-    const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
-    for (int i = threadIdx.x; i < r.I; i += RED_OUT * RED_SL) {
-        const int first = (i * r.row_tiles + rt) * n_chunks;
-        nks[i] = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
-    }
-    __syncthreads();
+// Sum of the partials of output m of one matrix that this thread's slice covers.
+// The (block, slot) pairs are numbered i * kmax + k and slice ks takes every
+// RED_SL-th of them, four at a time: slots that are not live (k beyond the number of
+// workgroups that touched this row tile of block i) are loaded from a live address
+// and masked, so the four loads never wait for one another or for the counts.
+__device__ __forceinline__ float slice_sum_any(const RedMat &r, int T, int t, int m, int rt, int n_chunks, int ks) {
+    const int total = r.I * r.kmax;
+    const int64_t stride = (int64_t)T * r.M;
+    const float *base = r.part + (int64_t)t * r.M + m;
     float acc = 0.f;
-    if (m < r.M) {
-        const int64_t stride = (int64_t)T * r.M;
-        for (int i = ks; i < r.I; i += RED_SL) {
-            const float *src = r.part + ((int64_t)i * r.kmax * T + t) * r.M + m;
-            const int nk = nks[i];
-            for (int k = 0; k < nk; k++) acc += src[k * stride];
-        }
-    }
-    red[ks][lo] = acc;
-    __syncthreads();
-    float s = 0.f;
-    if (ks == 0 && m < r.M) {
+    for (int s0 = ks; s0 < total; s0 += 4 * RED_SL) {
+        float v[4];
+        bool ok[4];
 #pragma unroll
-        for (int k = 0; k < RED_SL; k++) s += red[k][lo];
-        if (r.bias) s += (float)r.bias[m];
+        for (int j = 0; j < 4; j++) {
+            const int s = s0 + j * RED_SL;
+            const int sc = s < total ? s : ks;                 // slot ks exists whenever the loop runs
+            const int i = sc / r.kmax, k = sc - i * r.kmax;
+            const int first = (i * r.row_tiles + rt) * n_chunks;
+            const int nk = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
+            ok[j] = s < total && k < nk;
+            v[j] = base[(int64_t)(i * r.kmax + (k < nk ? k : 0)) * stride];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc += ok[j] ? v[j] : 0.f;
     }
-    __syncthreads();                             // nks / red are reused by a second call
-    return s;
+    return acc;
 }
 
 __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy,
     int rows_per_tile, int n_chunks) {
-    __shared__ int nks[RED_MAXBLOCKS];           // live partials of block i for this row tile
-    __shared__ float red[RED_SL][RED_OUT];
+    __shared__ float red[2][RED_SL][RED_OUT];
     const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
     int j = 0;
     if (grp.mode != EPI_SWIGLU) {
@@ -462,22 +465,34 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     const int local = blockIdx.x - r.first_block;
     const int per_t = (r.M + RED_OUT - 1) / RED_OUT;
     const int t = local / per_t, m0 = (local - t * per_t) * RED_OUT, m = m0 + lo;
-    const float s0 = reduce_partials(r, T, t, m0, rows_per_tile, n_chunks, nks, red);
-    if (grp.mode == EPI_SWIGLU) {
-        const float s1 = reduce_partials(grp.m[1], T, t, m0, rows_per_tile, n_chunks, nks, red);
-        if (ks == 0 && m < r.M) {
-            const float gate = (float)(half_t)s0, up = (float)(half_t)s1;
-            const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
-            y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
-        }
+    const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
+    const bool live = m < r.M;
+    const bool two = grp.mode == EPI_SWIGLU;
+    // residual and bias do not depend on the sums: fetch them before the reduction
+    float extra = 0.f, res = 0.f;
+    if (ks == 0 && live) {
+        if (r.bias) extra = (float)r.bias[m];
+        if (grp.mode == EPI_RESIDUAL) res = (float)residual[(int64_t)t * ldy + r.y_off + m];
+    }
+    red[0][ks][lo] = live ? slice_sum_any(r, T, t, m, rt, n_chunks, ks) : 0.f;
+    if (two) red[1][ks][lo] = live ? slice_sum_any(grp.m[1], T, t, m, rt, n_chunks, ks) : 0.f;
+    __syncthreads();
+    if (ks != 0 || !live) return;
+    float s0 = extra;
+#pragma unroll
+    for (int k = 0; k < RED_SL; k++) s0 += red[0][k][lo];
+    if (two) {
+        float s1 = grp.m[1].bias ? (float)grp.m[1].bias[m] : 0.f;
+#pragma unroll
+        for (int k = 0; k < RED_SL; k++) s1 += red[1][k][lo];
+        const float gate = (float)(half_t)s0, up = (float)(half_t)s1;
+        const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
+        y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
         return;
     }
-    if (ks == 0 && m < r.M) {
-        const int64_t at = (int64_t)t * ldy + r.y_off + m;
-        half_t v = (half_t)s0;
-        if (grp.mode == EPI_RESIDUAL) v = (half_t)((float)residual[at] + (float)v);
-        y[at] = v;
-    }
+    half_t v = (half_t)s0;
+    if (grp.mode == EPI_RESIDUAL) v = (half_t)(res + (float)v);
+    y[(int64_t)t * ldy + r.y_off + m] = v;
 }
 
 struct Plan {
