@@ -56,16 +56,17 @@ __global__ __launch_bounds__(RMS_THREADS) void rmsnorm_kernel(const half_t *__re
 // One workgroup per (query head, sequence).  256 threads = 16 groups of 16 lanes;
 // a group walks every 16th cached position, a lane owns 8 of the 128 dimensions
 // (one 16-byte load per cached row and lane, a row is one contiguous 256 bytes).
+// One pass: k and v of four positions are fetched together and folded into a
+// running (max, sum, weighted v) per group; the 16 groups are merged through LDS.
 constexpr int ATT_THREADS = 256, ATT_D = 128, ATT_MAX_LEN = 8192;
 
 __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     const half_t *__restrict__ qkv, half_t *__restrict__ kcache, half_t *__restrict__ vcache,
     const half_t *__restrict__ cosv, const half_t *__restrict__ sinv, const int64_t *__restrict__ pos_ptr,
     half_t *__restrict__ out, int heads, int kv_heads, int max_len) {
-    __shared__ float score[ATT_MAX_LEN];
     __shared__ float qs[ATT_D];                  // rotated query, pre-scaled
     __shared__ __attribute__((aligned(16))) half_t knew[ATT_D], vnew[ATT_D];   // this position's rotated k and v
-    __shared__ float red[ATT_THREADS / 64];
+    __shared__ float gm[16], gl[16];             // per group: running max, sum of exp
     __shared__ float accs[16][ATT_D];
     const int tid = threadIdx.x, lane16 = tid & 15, grp = tid >> 4;
     const int head = blockIdx.x, b = blockIdx.y;
@@ -75,6 +76,15 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     const half_t *kn = qkv + (int64_t)b * row + (heads + hk) * ATT_D;
     const half_t *vn = qkv + (int64_t)b * row + (heads + kv_heads + hk) * ATT_D;
     half_t *orow = out + ((int64_t)b * heads + head) * ATT_D;
+    // what does not depend on the position is fetched before the position is known
+    float qa = 0.f, qb = 0.f, ka = 0.f, kb = 0.f;
+    half_t vv = (half_t)0;
+    if (tid < ATT_D / 2) {
+        qa = (float)q[tid]; qb = (float)q[tid + ATT_D / 2];
+        ka = (float)kn[tid]; kb = (float)kn[tid + ATT_D / 2];
+    } else if (tid < ATT_D / 2 + ATT_D) {
+        vv = vn[tid - ATT_D / 2];
+    }
     const int64_t pos64 = *pos_ptr;
     if (pos64 < 0 || pos64 >= max_len) {         // nothing sensible to do: defined output, no access outside the cache
         if (tid < ATT_D) orow[tid] = (half_t)0;
@@ -86,15 +96,13 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
 
     if (tid < ATT_D / 2) {
         const float c = (float)cosv[(int64_t)pos * (ATT_D / 2) + tid], s = (float)sinv[(int64_t)pos * (ATT_D / 2) + tid];
-        const float qa = (float)q[tid], qb = (float)q[tid + ATT_D / 2];
         const float scale = 0.08838834764831845f;       // 1 / sqrt(128)
         qs[tid] = (float)(half_t)(qa * c - qb * s) * scale;
         qs[tid + ATT_D / 2] = (float)(half_t)(qb * c + qa * s) * scale;
-        const float ka = (float)kn[tid], kb = (float)kn[tid + ATT_D / 2];
         knew[tid] = (half_t)(ka * c - kb * s);
         knew[tid + ATT_D / 2] = (half_t)(kb * c + ka * s);
     } else if (tid < ATT_D / 2 + ATT_D) {
-        vnew[tid - ATT_D / 2] = vn[tid - ATT_D / 2];
+        vnew[tid - ATT_D / 2] = vv;
     }
     __syncthreads();
     if (head % rep == 0 && tid < ATT_D) {        // one head of the group appends to the cache
@@ -105,53 +113,57 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     float qreg[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) qreg[e] = qs[8 * lane16 + e];
-    for (int p = grp; p <= pos; p += 16) {
-        const half8_t k8 = p == pos ? *reinterpret_cast<const half8_t *>(knew + 8 * lane16)
-                                    : *reinterpret_cast<const half8_t *>(kc + (int64_t)p * ATT_D + 8 * lane16);
+    float m = -INFINITY, l = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    auto score_of = [&](const half8_t k8) {
         float d = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; e++) d += qreg[e] * (float)k8[e];
 #pragma unroll
         for (int o = 8; o >= 1; o >>= 1) d += __shfl_xor(d, o, 64);
-        if (lane16 == 0) score[p] = d;
-    }
-    __syncthreads();
-
-    float mx = -INFINITY;
-    for (int p = tid; p <= pos; p += ATT_THREADS) mx = fmaxf(mx, score[p]);
+        return d;                                 // the same value in all 16 lanes of the group
+    };
+    auto fold = [&](float sc, const half8_t v8) {
+        const float mn = fmaxf(m, sc);
+        const float r = __expf(m - mn), w = __expf(sc - mn);      // exp(-inf) = 0 on the first position
+        l = l * r + w;
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    if ((tid & 63) == 0) red[tid >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    float sum = 0.f;
-    for (int p = tid; p <= pos; p += ATT_THREADS) {
-        const float e = __expf(score[p] - mx);
-        score[p] = e;
-        sum += e;
-    }
-    sum = wave_sum(sum);
-    if ((tid & 63) == 0) red[tid >> 6] = sum;
-    __syncthreads();
-    const float inv = 1.f / (red[0] + red[1] + red[2] + red[3]);
-
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int p = grp; p <= pos; p += 16) {
-        const half8_t v8 = p == pos ? *reinterpret_cast<const half8_t *>(vnew + 8 * lane16)
-                                    : *reinterpret_cast<const half8_t *>(vc + (int64_t)p * ATT_D + 8 * lane16);
-        const float w = (float)(half_t)(score[p] * inv);      // probabilities rounded to fp16 before the product
+        for (int e = 0; e < 8; e++) acc[e] = acc[e] * r + w * (float)v8[e];
+        m = mn;
+    };
+    for (int p0 = grp; p0 < pos; p0 += 64) {
+        half8_t k8[4], v8[4];
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += w * (float)v8[e];
+        for (int j = 0; j < 4; j++) {
+            const int p = min(p0 + 16 * j, pos - 1);
+            k8[j] = *reinterpret_cast<const half8_t *>(kc + (int64_t)p * ATT_D + 8 * lane16);
+            v8[j] = *reinterpret_cast<const half8_t *>(vc + (int64_t)p * ATT_D + 8 * lane16);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float sc = score_of(k8[j]);
+            if (p0 + 16 * j < pos) fold(sc, v8[j]);
+        }
     }
+    if (grp == 0)      // this step's own k and v, from LDS
+        fold(score_of(*reinterpret_cast<const half8_t *>(knew + 8 * lane16)),
+             *reinterpret_cast<const half8_t *>(vnew + 8 * lane16));
+    if (lane16 == 0) { gm[grp] = m; gl[grp] = l; }
 #pragma unroll
     for (int e = 0; e < 8; e++) accs[grp][8 * lane16 + e] = acc[e];
     __syncthreads();
     if (tid < ATT_D) {
-        float o = 0.f;
+        float mx = gm[0];
 #pragma unroll
-        for (int gq = 0; gq < 16; gq++) o += accs[gq][tid];
-        orow[tid] = (half_t)o;
+        for (int gq = 1; gq < 16; gq++) mx = fmaxf(mx, gm[gq]);
+        float o = 0.f, den = 0.f;
+#pragma unroll
+        for (int gq = 0; gq < 16; gq++) {
+            const float r = gl[gq] > 0.f ? __expf(gm[gq] - mx) : 0.f;     // groups that saw no position
+            o += r * accs[gq][tid];
+            den += r * gl[gq];
+        }
+        orow[tid] = (half_t)(o / den);
     }
 }
 

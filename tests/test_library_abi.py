@@ -83,3 +83,39 @@ def test_workspace_bytes(L):
     for T in (1, 4, 8):
         b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
         assert b > 0 and b % (T * 4096 * 4) == 0 and b < 4096 * 4096 * 2
+
+
+def test_group_and_decode_step_validation(L):
+    nul, one, odd = ctypes.c_void_p(0), ctypes.c_void_p(256), ctypes.c_void_p(257)
+    mats = (_lib.bs_matrix * 2)()
+    for m in mats:
+        m.packed, m.u, m.vt, m.bias, m.I, m.M = 256, 256, 256, None, 2, 128
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 1) > 0
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 500, 16, 1) == -2          # N % 8
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 520, 16, 1) == -2          # not a decode-kernel shape
+    assert L.bs_forward_group_workspace_bytes(mats, 5, 512, 16, 1) == -2          # more than BS_MAX_GROUP
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 9) == -2          # more than 8 tokens
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 17, 1) == -3
+    assert L.bs_forward_group_workspace_bytes(nul, 2, 512, 16, 1) == -1
+    big = 1 << 30
+    assert L.bs_forward_group(mats, 2, 512, 16, nul, 1, 0, nul, one, one, big, nul) == -1       # x
+    assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 1, nul, one, one, big, nul) == -1       # residual epilogue, no residual
+    assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 7, nul, one, one, big, nul) == -2       # unknown epilogue
+    assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 0, nul, one, nul, 0, nul) == -5
+    mats[1].vt = 257
+    assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 0, nul, one, one, big, nul) == -4
+    mats[1].vt = 256
+    mats[1].M = 64
+    assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 2, nul, one, one, big, nul) == -2       # SwiGLU needs equal M
+    # rmsnorm / attention
+    assert L.bs_rmsnorm_f16(one, one, one, 1, 100, 1e-5, nul) == -2
+    assert L.bs_rmsnorm_f16(one, one, one, 1, 32768, 1e-5, nul) == -2
+    assert L.bs_rmsnorm_f16(one, nul, one, 1, 512, 1e-5, nul) == -1
+    assert L.bs_rmsnorm_f16(odd, one, one, 1, 512, 1e-5, nul) == -4
+    assert L.bs_rmsnorm_f16(nul, nul, nul, 0, 512, 1e-5, nul) == 0
+    att = lambda *a: L.bs_attention_decode_f16(*a)
+    assert att(one, one, one, one, one, one, one, 1, 32, 8, 64, 128, nul) == -2                 # head_dim
+    assert att(one, one, one, one, one, one, one, 1, 32, 5, 128, 128, nul) == -2                # heads % kv_heads
+    assert att(one, one, one, one, one, one, one, 1, 32, 8, 128, 10000, nul) == -2              # max_len
+    assert att(one, one, one, one, one, nul, one, 1, 32, 8, 128, 128, nul) == -1                # pos
+    assert att(one, odd, one, one, one, one, one, 1, 32, 8, 128, 128, nul) == -4
