@@ -50,6 +50,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
+    ap.add_argument("--only", choices=["decode_8b", "prefill"], default=None,
+                    help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
     return ap.parse_args()
 
@@ -224,6 +226,28 @@ def main():
                          for j in range(len(fns))]          # ms per forward
         return wall, per_layer
 
+    def prefill_side(detail):
+        pre = {}
+        for T in PREFILL_T:
+            lp = build_sweep(T, blocks=[8])
+            _, perp = time_sweep(lp, 3, 1, per_layer_events=True)
+            useful = sum(2.0 * L.M * L.N * L.T + 2.0 * 16 * L.I * L.M * L.N for L in lp)
+            tp = sum(perp) * 1e-3
+            pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
+                            "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+            detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
+                        "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
+                       for L, ms in zip(lp, perp)]
+            del lp
+        return pre
+
+    if a.only == "decode_8b":
+        print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
+        return
+    if a.only == "prefill":
+        print(json.dumps({"prefill": prefill_side([])}))
+        return
+
     # ---------------------------------------------------------------- headline: T = 1 sweep
     layers = build_sweep(1)
     pass_bytes = sum(L.bytes for L in layers)
@@ -294,18 +318,7 @@ def main():
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l4, per4)]
         del l4
         # ------------------------------------------------------------ prefill (useful flops)
-        pre = {}
-        for T in PREFILL_T:
-            lp = build_sweep(T, blocks=[8])
-            _, perp = time_sweep(lp, 3, 1, per_layer_events=True)
-            useful = sum(2.0 * L.M * L.N * L.T + 2.0 * 16 * L.I * L.M * L.N for L in lp)
-            tp = sum(perp) * 1e-3
-            pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
-                            "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
-            detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
-                        "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
-                       for L, ms in zip(lp, perp)]
-            del lp
+        pre = prefill_side(detail)
         out["prefill"] = pre
 
     if not a.no_extras:
