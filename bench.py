@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
-    ap.add_argument("--only", choices=["decode_8b", "prefill"], default=None,
+    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
     return ap.parse_args()
@@ -98,6 +98,38 @@ def cpu_baseline(layers_cpu):
             "sample": f"the T=1 sweep restricted to blocks {{1,2,4}} on all four shapes ({len(layers_cpu)} layers, "
                       f"{tot_b / 1e6:.0f} MB algorithmic, {tot_t:.1f} s) through the level-0 torch-CPU restatement",
             "seconds": round(tot_t, 2)}
+
+
+def e2e_decode_70b(torch, dev, batch=8, prompt_len=16, new_tokens=64):
+    """Random-init Llama-3.1-70B-shape decode, `batch` sequences in lock step (every
+    linear sees 8 tokens: two passes of four through the decode kernel), about 30 GB
+    of weights.  The prompt is fed token by token (prefill is not what is measured)."""
+    from bitstack_amd.utils.llama_decode import LLAMA_70B, SyntheticLlamaDecoder, synthetic_compression_config
+    cfg, total = synthetic_compression_config(LLAMA_70B, 30e9, lo=1, hi=8)
+    model = SyntheticLlamaDecoder(LLAMA_70B, cfg, prompt_len + new_tokens + 8, dev, batch=batch)
+    prompt = torch.randint(0, LLAMA_70B.vocab, (batch, prompt_len), generator=torch.Generator().manual_seed(0)).to(dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        model.prefill_positions(prompt, fused=True)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        model.step_fused()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(new_tokens):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    wbytes = model.weight_bytes()
+    blocks = list(cfg.values())
+    return {"tok_s": round(batch * new_tokens / dt, 1), "ms_per_step": round(dt / new_tokens * 1e3, 3), "batch": batch,
+            "weight_GB": round(wbytes / 1e9, 2), "blocks_per_linear_mean": round(sum(blocks) / len(blocks), 2),
+            "hbm_roofline_tok_s": round(batch * 8e12 / wbytes, 1),
+            "config": f"80 layers, hidden 8192, inter 28672, 64Q/8KV, vocab 128256, batch {batch}, {prompt_len}-token prompt, "
+                      f"{new_tokens} greedy tokens per sequence, fused step, one HIP-graph replay per step"}
 
 
 def e2e_decode(torch, dev, prompt_len=128, new_tokens=256):
@@ -243,6 +275,9 @@ def main():
 
     if a.only == "decode_8b":
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
+        return
+    if a.only == "decode_70b":
+        print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev)}))
         return
     if a.only == "prefill":
         print(json.dumps({"prefill": prefill_side([])}))
