@@ -93,11 +93,23 @@ __constant__ float step_mid_table[16] = {0.f, 1.f, 5.f, 9.f, 17.f, 33.f, 65.f, 1
 // LDS image of Z for one chunk: [t][step (16)][g (4)][r (16)][slot (8)] halves.
 __device__ inline int z_index(int t, int st, int g, int r) { return (((t * 16 + st) * 4 + g) * 16 + r) * 8; }
 
-__device__ inline uint32_t and_or(uint32_t w, uint32_t mask, uint32_t base) {
-    uint32_t d;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(w), "s"(mask), "v"(base));
-    return d;
+// (w & mask) | base as ONE v_and_or_b32.  VOP3 takes no literal and one scalar
+// operand, so the two constants are first pinned into registers (mask scalar, base
+// vector) with empty asm statements the optimiser cannot see through; the merge
+// itself stays an ordinary expression.  It must not be written as an asm
+// instruction: the compiler's hazard recogniser does not look inside inline asm,
+// and a VALU write to registers that an MFMA issued just before still reads as its
+// accumulator input (the MFMA reads SrcC several cycles after issue) corrupts that
+// MFMA unless the recogniser can see the write and pad it.
+__device__ inline uint32_t pin_scalar(uint32_t v) {
+    asm("" : "+s"(v));
+    return v;
 }
+__device__ inline uint32_t pin_vector(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
+__device__ inline uint32_t and_or(uint32_t w, uint32_t mask, uint32_t base) { return (w & mask) | base; }
 
 // One producer item: rank r, lane group pg, word p, byte pair (JB, JB + 2) of
 // the word.  Two 16-byte pieces of vt (8 consecutive columns each) times x
@@ -271,12 +283,13 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
                 for (int jr = 0; jr < R; jr++) w[jr] = w[jr] << 2;
             }
             constexpr int j = step_pos(st);
-            constexpr uint32_t mask = 0x00010001u << j;
+            constexpr uint32_t mask_c = 0x00010001u << j;
+            const uint32_t mask = pin_scalar(mask_c), base = j == 14 ? 0u : pin_vector(pos_base(j));
 #pragma unroll
             for (int jr = 0; jr < R; jr++) {
                 uint4_t sb;
 #pragma unroll
-                for (int p = 0; p < 4; p++) sb[p] = (j == 14) ? (w[jr][p] & mask) : and_or(w[jr][p], mask, pos_base(j));
+                for (int p = 0; p < 4; p++) sb[p] = (j == 14) ? (w[jr][p] & mask) : and_or(w[jr][p], mask, base);
                 const half8_t sf = __builtin_bit_cast(half8_t, sb);
 #pragma unroll
                 for (int t = 0; t < T; t++)

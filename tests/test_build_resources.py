@@ -19,7 +19,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not available")
-@pytest.mark.parametrize("src", ["gemv.hip", "gemm.hip", "reconstruct.hip", "pack.hip"])
+@pytest.mark.parametrize("src", ["gemv.hip", "gemm.hip", "reconstruct.hip", "pack.hip", "decode_step.hip"])
 def test_no_spill_code_in_loops_and_little_scratch(src, tmp_path):
     asm = tmp_path / "k.s"
     out = subprocess.run([HIPCC] + FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", str(asm)],
@@ -40,3 +40,19 @@ def test_no_spill_code_in_loops_and_little_scratch(src, tmp_path):
     assert not offenders, f"spill code inside a loop: {offenders[:4]}"
     sizes = re.findall(r"\.private_segment_fixed_size:\s+(\d+)", asm.read_text())
     assert sizes and max(int(v) for v in sizes) <= 64, f"scratch bytes per lane: {sorted(set(sizes))}"
+
+
+def test_no_instruction_is_written_as_inline_asm():
+    """hipcc's hazard recogniser does not look inside inline asm: a VALU instruction
+    written that way next to MFMAs can overwrite registers an in-flight MFMA still
+    reads (met with v_and_or_b32: one row tile in four came out wrong once register
+    allocation changed).  Only empty asm statements (register pinning) are allowed."""
+    offenders = []
+    for name in sorted(os.listdir(CSRC)):
+        if not name.endswith((".hip", ".h")):
+            continue
+        text = open(os.path.join(CSRC, name)).read()
+        for m in re.finditer(r"\basm\s*(?:volatile)?\s*\(\s*\"([^\"]*)\"", text):
+            if m.group(1).strip():
+                offenders.append((name, m.group(1)))
+    assert not offenders, offenders
