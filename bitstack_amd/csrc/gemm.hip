@@ -5,21 +5,24 @@
 // row (A = tokens) or one column (B = features), i.e. one 16-byte read per
 // fragment.
 //
-// More than 128 tokens: linear_f16_kernel, 2 x 2 waves of 2 x 2 MFMA tiles
-// (128 tokens x 128 features per workgroup), k-steps of 64 columns through LDS;
-// rows are padded by 8 halves so that the eight lanes served per LDS cycle hit
-// disjoint banks.  Global loads for step s+1 are issued before the MFMAs of
-// step s (register staging, two LDS buffers, one barrier per step).  Larger
-// per-wave tiles (4 x 2, 2 x 4) and 32-column steps measured slower: with one
-// step of look-ahead the kernel is bound by load latency, not by LDS traffic.
+// More than 128 tokens: linear_f16_kernel, 2 x 2 (or 2 x 4) waves of 2 x 2 MFMA tiles
+// (128 tokens x 128 or 256 features per workgroup), k-steps of 64 columns through
+// LDS; rows are padded by 8 halves so that the eight lanes served per LDS cycle hit
+// disjoint banks.  Global loads run two k-steps ahead of the MFMAs through two
+// register sets, all of them unconditional with a scalar base and a 32-bit lane
+// offset (no address arithmetic or selects in the loop); two LDS buffers, one
+// barrier per step.  Measured dead ends: 32-column steps, 128 x 64 and 128 x 128
+// per-wave tiles (the compiler's register allocation collapses), 256 x 256
+// workgroup tiles with 16 waves.
 // 33..128 tokens use narrower workgroups of the same kernel (more workgroups for
 // the few token rows); up to 32 tokens: linear_skinny_kernel (below).
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
 
-template <int WT, int WF, int AT, int AF, int GK>
+template <int WT, int WF, int AT, int AF, int GK, bool KTAIL>
 __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     const half_t *__restrict__ x, const half_t *__restrict__ w, const half_t *__restrict__ bias,
     half_t *__restrict__ y, int T, int M, int N) {
@@ -28,8 +31,9 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     constexpr int ROWS = BT + BF;                            // LDS rows per buffer (x rows, then w rows)
     constexpr int PPR = GK / 8;                              // 16-byte pieces per row and k-step
     constexpr int LSTRIDE = GK + 8;                          // halves per LDS row (padded)
-    constexpr int PIECES = ROWS * PPR;                       // 16-byte pieces per k-step
-    constexpr int PER_THREAD = (PIECES + THREADS - 1) / THREADS;
+    constexpr int JX = BT * PPR / THREADS, JW = BF * PPR / THREADS;   // pieces per thread: x rows, w rows
+    static_assert(BT * PPR % THREADS == 0 && BF * PPR % THREADS == 0, "every thread stages whole pieces");
+    constexpr int PER_THREAD = JX + JW;
     extern __shared__ __attribute__((aligned(16))) half_t lds_raw[];
     half_t (*lds)[ROWS * (GK + 8)] = reinterpret_cast<half_t (*)[ROWS * (GK + 8)]>(lds_raw);
 
@@ -38,17 +42,23 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     const int wt = (wave / WF) * (AT * 32), wf = (wave % WF) * (AF * 32);
     const int l32 = lane & 31, kh = lane >> 5;
 
-    // loader role: piece p = tid + THREADS * j -> LDS row p / PPR, 16-byte piece p % PPR
-    const half_t *src[PER_THREAD];
+    // Loader role.  Piece j of a thread is row tid / PPR + (THREADS / PPR) * j of the x
+    // tile (j < JX) or of the w tile, 16-byte piece tid % PPR.  Addresses are a
+    // workgroup-uniform pointer (tile origin + k-step, scalar registers) plus a 32-bit
+    // per-thread byte offset; rows beyond T or M repeat the last row (their outputs are
+    // never stored), so no load in the main loop is conditional.
+    const char *xt = reinterpret_cast<const char *>(x + (int64_t)t0 * N);
+    const char *wt_ = reinterpret_cast<const char *>(w + (int64_t)m0 * N);
+    const int lrow = tid / PPR, lpiece = tid % PPR;
+    uint32_t off[PER_THREAD];
     int dst[PER_THREAD];
-    bool live[PER_THREAD];
 #pragma unroll
     for (int j = 0; j < PER_THREAD; j++) {
-        const int p = tid + THREADS * j, row = p / PPR, piece = p % PPR;
-        live[j] = p < PIECES;
-        const int r = live[j] ? row : 0;
-        src[j] = (r < BT ? x + (int64_t)min(t0 + r, T - 1) * N : w + (int64_t)min(m0 + r - BT, M - 1) * N) + 8 * piece;
-        dst[j] = r * LSTRIDE + 8 * piece;
+        const bool isx = j < JX;
+        const int r = lrow + (THREADS / PPR) * (isx ? j : j - JX);
+        const int rr = isx ? min(r, T - 1 - t0) : min(r, M - 1 - m0);
+        off[j] = (uint32_t)rr * (uint32_t)N * 2u + 16u * lpiece;
+        dst[j] = ((isx ? 0 : BT) + r) * LSTRIDE + 8 * lpiece;
     }
 
     float16_t acc[AT][AF];
@@ -60,27 +70,37 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
             for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
 
     const int steps = (N + GK - 1) / GK;
-    uint4_t stage[PER_THREAD];
-    auto fetch = [&](int step) {
+    // Two register sets: while step s is multiplied, the pieces of step s + 1 are already
+    // in one set (in flight or landed) and those of step s + 2 are requested into the other.
+    // Every request is unconditional (past the end the last step is requested again), so
+    // the compiler's count of outstanding loads is exact and a wait for one set never
+    // drains the other.  KTAIL (N not a multiple of GK): pieces beyond column N are read
+    // from column 0 instead and replaced by zeros.
+    uint4_t stage[2][PER_THREAD];
+    auto fetch = [&](auto setc, int step_) {
+        constexpr int set = decltype(setc)::value;
+        const int step = min(step_, steps - 1);
+        if constexpr (KTAIL) {
+            const bool in = step * GK + 8 * lpiece < N;              // N % 8 == 0: a piece is all in or all out
+            const uint32_t koff = in ? (uint32_t)step * (GK * 2) : 0u - 16u * lpiece;
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; j++) {
-            const int piece = (tid + THREADS * j) % PPR;
-            const bool in = live[j] && step * GK + 8 * piece < N;     // N % 8 == 0: a piece is all in or all out
-            stage[j] = in ? *reinterpret_cast<const uint4_t *>(src[j] + step * GK) : (uint4_t){0, 0, 0, 0};
+            for (int j = 0; j < PER_THREAD; j++) {
+                const uint4_t v = *reinterpret_cast<const uint4_t *>((j < JX ? xt : wt_) + (off[j] + koff));
+                stage[set][j] = in ? v : (uint4_t){0, 0, 0, 0};
+            }
+        } else {
+            const char *xs = xt + (int64_t)step * (GK * 2), *ws = wt_ + (int64_t)step * (GK * 2);
+#pragma unroll
+            for (int j = 0; j < PER_THREAD; j++)
+                stage[set][j] = *reinterpret_cast<const uint4_t *>((j < JX ? xs : ws) + off[j]);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](auto setc, int buf) {
+        constexpr int set = decltype(setc)::value;
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; j++)
-            if (live[j]) *reinterpret_cast<uint4_t *>(&lds[buf][dst[j]]) = stage[j];
+        for (int j = 0; j < PER_THREAD; j++) *reinterpret_cast<uint4_t *>(&lds[buf][dst[j]]) = stage[set][j];
     };
-
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int step = 0; step < steps; step++) {
-        const int buf = step & 1;
-        if (step + 1 < steps) fetch(step + 1);
+    auto multiply = [&](int buf) {
         const half_t *xs = &lds[buf][0], *ws = &lds[buf][BT * LSTRIDE];
 #pragma unroll
         for (int kk = 0; kk < GK / 16; kk++) {
@@ -97,8 +117,24 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
                 for (int bi = 0; bi < AF; bi++)
                     acc[ai][bi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ai], b[bi], acc[ai][bi], 0, 0, 0);
         }
-        if (step + 1 < steps) stash(buf ^ 1);
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    // step s reads LDS buffer s & 1; its pieces travelled through register set s & 1
+    auto one_step = [&](auto cur, auto nxt, int step) {
+        fetch(cur, step + 2);                                 // set `cur` was emptied into LDS a step ago
+        multiply(step & 1);
+        stash(nxt, (step + 1) & 1);                           // after the last step: a copy nobody reads
         __syncthreads();
+    };
+
+    fetch(S0{}, 0);
+    fetch(S1{}, 1);
+    stash(S0{}, 0);
+    __syncthreads();
+    for (int step = 0; step < steps; step += 2) {
+        one_step(S0{}, S1{}, step);
+        if (step + 1 < steps) one_step(S1{}, S0{}, step + 1);
     }
 
     // D[token, feature]: lane holds feature l32, tokens 8 * (v / 4) + 4 * kh + v % 4
@@ -208,12 +244,17 @@ int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y
     constexpr size_t lds = (size_t)2 * (BT + BF) * (GK + 8) * sizeof(half_t);
     static bool raised = false;
     if (lds > 64 * 1024 && !raised) {
-        BS_HIP_TRY(hipFuncSetAttribute((const void *)linear_f16_kernel<WT, WF, AT, AF, GK>,
+        BS_HIP_TRY(hipFuncSetAttribute((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        BS_HIP_TRY(hipFuncSetAttribute((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
     dim3 grid((unsigned)bs_cdiv(M, BF), (unsigned)bs_cdiv(T, BT));
-    linear_f16_kernel<WT, WF, AT, AF, GK><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
+    if (N % GK == 0)
+        linear_f16_kernel<WT, WF, AT, AF, GK, false><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
+    else
+        linear_f16_kernel<WT, WF, AT, AF, GK, true><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
     return BS_OK;
 }
 
@@ -229,7 +270,9 @@ int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, h
             st = M >= 8192 ? launch_tiled<2, 2, 2, 1, 64>(x, w, bias, y, T, M, N, s)
                            : launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
         } else {
-            st = launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+            // 128 x 256 tiles (8 waves) once they still give every CU a workgroup, else 128 x 128
+            st = bs_cdiv(T, 128) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s)
+                                                             : launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
         }
         if (st != BS_OK) return st;
     } else {
