@@ -5,8 +5,8 @@
 // Tiled kernel.  A workgroup owns a strip of 128 columns and a range of rows.
 // It first stages the strip's slice of vt for ALL blocks in LDS, transposed to
 // [block][column][rank] (vt is stored rank-major, the MFMA wants the rank
-// index contiguous per lane; column stride 18 halves keeps the 8-byte fragment
-// reads off each other's banks), then walks its rows 16 per wave at a time with
+// index contiguous per lane; column stride 20 halves keeps the 8-byte fragment
+// reads aligned and off each other's banks), then walks its rows 16 per wave at a time with
 // no further barrier.  Per block the rank-k product of a 16 x 16 patch is one
 // v_mfma_f32_16x16x16_f16 computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
 // so that a lane ends up with four consecutive columns of one row - exactly
@@ -18,11 +18,11 @@
 namespace {
 
 constexpr int RT_COLS = 128;   // columns per workgroup strip
-constexpr int VSTRIDE = 18;    // halves between consecutive columns in LDS
-constexpr int RT_MAXB = 32;    // most blocks whose vt strip fits in LDS (32 x 4.5 KB)
+constexpr int VSTRIDE = 20;    // halves between consecutive columns in LDS (8-byte aligned fragments)
+constexpr int RT_MAXB = 30;    // most blocks whose vt strip fits in LDS (30 x 5 KB)
 
 template <bool PACKED>
-__global__ __launch_bounds__(256) void reconstruct_tile_kernel(
+__global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
     const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
     const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
     int I, int M, int N, int K, int rows_per_wg) {
@@ -30,8 +30,21 @@ __global__ __launch_bounds__(256) void reconstruct_tile_kernel(
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * RT_COLS;
-    const int row_begin = blockIdx.y * rows_per_wg;
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  The eight
+    // strips that share one 128-byte line of sign bytes must meet in ONE L2, and so
+    // should the row groups that re-read one strip of vt: every XCD gets a contiguous
+    // run of slots ordered (octet of strips, row group, strip within the octet).  The
+    // grid is padded to whole octets; slots beyond the last strip do nothing.
+    int n0, row_begin;
+    {
+        const int nb = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
+        const int xcd = lin & 7, loc = lin >> 3, base = nb >> 3, rem = nb & 7;
+        const int v = xcd * base + min(xcd, rem) + loc;
+        const int rest = v >> 3, strip = (rest / (int)gridDim.y) * 8 + (v & 7);
+        if (strip * RT_COLS >= N) return;
+        n0 = strip * RT_COLS;
+        row_begin = (rest % (int)gridDim.y) * rows_per_wg;
+    }
     const int row_end = min(row_begin + rows_per_wg, M);
     const int64_t row_bytes = N >> 3;
     const int64_t block_bytes = (int64_t)M * row_bytes;
@@ -82,9 +95,7 @@ __global__ __launch_bounds__(256) void reconstruct_tile_kernel(
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
                     const half_t *ap = vb + (16 * s + lm) * VSTRIDE + 4 * g;
-                    half2_t a01 = *reinterpret_cast<const half2_t *>(ap);
-                    half2_t a23 = *reinterpret_cast<const half2_t *>(ap + 2);
-                    half4_t a = {a01[0], a01[1], a23[0], a23[1]};
+                    const half4_t a = *reinterpret_cast<const half4_t *>(ap);
                     float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     if (PACKED) {
                         uint32_t t = swc[s >> 1] << (sh_even - 16 * (s & 1));
@@ -155,12 +166,17 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
     const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && bs_aligned(vt, 16) && bs_aligned(w, 8) &&
                        bs_aligned(u, 8) && (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
     if (tiled) {
-        // about four workgroups per CU; every workgroup re-stages its vt strip, so rows
-        // per workgroup stay a multiple of 64 and not too small
-        const int strips = N / RT_COLS;
-        int row_groups = (int)bs_cdiv(1024, strips);
+        // One wave of workgroups: as many row groups as the resident slots allow (LDS decides
+        // how many workgroups a CU holds), so that no second, partial wave trails behind.
+        // Every workgroup re-stages its vt strip, so rows per workgroup stay a multiple of 64.
+        const int strips = N / RT_COLS, strips8 = (int)bs_cdiv(strips, 8) * 8;
+        const size_t lds_need = (size_t)I * RT_COLS * VSTRIDE * sizeof(half_t);
+        int per_cu = (int)((160 * 1024) / lds_need);
+        if (per_cu > 8) per_cu = 8;
+        if (per_cu < 1) per_cu = 1;
+        int row_groups = (256 * per_cu) / strips8;
+        if (row_groups < 1) row_groups = 1;
         int rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
-        if (rows_per_wg < 128) rows_per_wg = 128;
         row_groups = (int)bs_cdiv(M, rows_per_wg);
         const size_t lds = (size_t)I * RT_COLS * VSTRIDE * sizeof(half_t);
         static size_t raised = 0;
@@ -169,7 +185,7 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             raised = lds;
         }
-        dim3 grid(strips, row_groups);
+        dim3 grid((unsigned)bs_cdiv(strips, 8) * 8, row_groups);
         reconstruct_tile_kernel<PACKED><<<grid, 256, lds, s>>>(packed, sign, u, vt, w, I, M, N, K, rows_per_wg);
     } else {
         int64_t blocks = bs_cdiv((int64_t)M * N, 256);
