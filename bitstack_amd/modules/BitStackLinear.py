@@ -217,3 +217,39 @@ class BitStackLinear(nn.Module):
                 delattr(self, f"qweight_{i}")
             delattr(self, f"u_{i}")
             delattr(self, f"vt_{i}")
+
+    # ---- beyond the reference: blocks that really come and go ----------------
+    # The reference's pop_one_bit / add_one_bit only move a counter
+    # (BitStackLinear.py:173-178); these two move memory, on the stacked layout.
+    def trim_blocks(self):
+        """Give back the memory of the stacked blocks beyond w_bit."""
+        if not hasattr(self, "u") or self.u is None or self.u.shape[0] <= self.w_bit:
+            return 0
+        per_block = self.u[0].numel() * 2 + self.vt[0].numel() * 2 + (0 if self.no_avd else self.qweight[0].numel())
+        freed = (self.u.shape[0] - self.w_bit) * per_block
+        keep = self.w_bit
+        self.u = self.u[:keep].clone()
+        self.vt = self.vt[:keep].clone()
+        if not self.no_avd:
+            self.qweight = self.qweight[:keep].clone()
+        return freed
+
+    def append_blocks(self, qweight, u, vt):
+        """Stack further blocks ([n, M*N/8] uint8, [n, M, k], [n, k, N] fp16) behind the
+        loaded ones and count them in."""
+        if not hasattr(self, "u") or self.u is None:
+            raise RuntimeError("append_blocks works on the stacked layout: call stack_blocks() first")
+        if self.w_bit != self.u.shape[0]:
+            raise RuntimeError("blocks beyond w_bit are still stacked: trim_blocks() first")
+        n = u.shape[0]
+        if u.shape[1:] != self.u.shape[1:] or vt.shape[1:] != self.vt.shape[1:] or vt.shape[0] != n:
+            raise ValueError("block shapes do not match the layer")
+        dev = self.u.device
+        self.u = torch.cat([self.u, u.to(dev, torch.float16)])
+        self.vt = torch.cat([self.vt, vt.to(dev, torch.float16)])
+        if not self.no_avd:
+            if qweight is None or qweight.shape != (n, self.qweight.shape[1]) or qweight.dtype != torch.uint8:
+                raise ValueError("packed signs do not match the layer")
+            self.qweight = torch.cat([self.qweight, qweight.to(dev)])
+        self.w_bit += n
+

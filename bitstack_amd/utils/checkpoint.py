@@ -158,6 +158,47 @@ def load_bitstack_checkpoint(path, compression_config=None, niter=None, device="
     return linears, other
 
 
+def apply_compression_config(path, linears, compression_config):
+    """Move already loaded modules (stacked layout) to another compression config of
+    the same checkpoint: layers that get fewer blocks drop and free the surplus,
+    layers that get more read just the missing blocks from disk.  What the
+    reference's set_model_bits (model_utils.py:11-17) does with a counter, done
+    with memory.  Returns (bytes_freed, bytes_loaded)."""
+    wmap = _weight_map(path)
+    shards = _Shards(path, wmap)
+    freed = loaded = 0
+    try:
+        for lname, mod in linears.items():
+            want = compression_config[lname]
+            if want < 1:
+                raise ValueError(f"{lname}: at least one block is needed, got {want}")
+            have = mod.w_bit
+            if want < have:
+                mod.set_bit(want)
+                freed += (have - want) * mod.memory_per_bit()
+                mod.trim_blocks()
+            elif want > have:
+                if mod.u.shape[0] > have:          # surplus blocks still stacked from an earlier set_bit
+                    mod.trim_blocks()
+                _, layer, name = lname.split(".", 2)
+                base = next((k[: k.rfind(".")] for k in wmap
+                             if _BLOCK_KEY.match(k) and k.endswith(f"layers.{layer}.{name}.u_0")), None)
+                if base is None:
+                    raise KeyError(f"{lname} is not in the checkpoint")
+                idx = range(have, want)
+                missing = [f"{base}.{kind}_{i}" for i in idx for kind in ("u", "vt") if f"{base}.{kind}_{i}" not in wmap]
+                if missing:
+                    raise KeyError(f"{lname}: checkpoint lacks {missing[:4]}")
+                u = torch.stack([shards.get(f"{base}.u_{i}") for i in idx])
+                vt = torch.stack([shards.get(f"{base}.vt_{i}") for i in idx])
+                q = None if mod.no_avd else torch.stack([shards.get(f"{base}.qweight_{i}") for i in idx])
+                mod.append_blocks(q, u, vt)
+                loaded += (want - have) * mod.memory_per_bit()
+    finally:
+        shards.close()
+    return freed, loaded
+
+
 def save_bitstack_checkpoint(path, linears, other=None, compression_configs=None, max_shard_bytes=None,
                              key_prefix="model.layers."):
     """Writes `linears` ({"layer.{L}.{name}": BitStackLinear}, stacked or not) and

@@ -127,3 +127,52 @@ def test_save_then_load_round_trip(tmp_path, max_shard_bytes):
             assert torch.equal(getattr(again[k], attr), getattr(linears[k], attr))
         assert (again[k].bias is None) == (linears[k].bias is None)
     assert ck.read_compression_configs(str(out)) == [{"memory": 1, "layers": {}}]
+
+
+def test_blocks_really_come_and_go(tmp_path):
+    tensors = _write(tmp_path, blocks=3, shards=3)
+    names = [f"layer.{L}.{n}" for L in range(2) for n in PROJ]
+    linears, _ = ck.load_bitstack_checkpoint(str(tmp_path), niter=2, device="cpu", fused_level=5, dense=False)
+    x = {n: torch.randn(2, linears[n].in_features, generator=torch.Generator().manual_seed(3)).half() for n in names}
+
+    def dense_out(name, blocks):
+        _, L, proj = name.split(".", 2)
+        base = f"model.layers.{L}.{proj}"
+        packed = np.stack([tensors[f"{base}.qweight_{i}"].numpy() for i in range(blocks)])
+        u = np.stack([tensors[f"{base}.u_{i}"].numpy() for i in range(blocks)])
+        vt = np.stack([tensors[f"{base}.vt_{i}"].numpy() for i in range(blocks)])
+        bias = tensors.get(f"{base}.bias")
+        return bo.forward_exact(packed, u, vt, x[name].numpy(), None if bias is None else bias.numpy())
+
+    # down to one block in some layers, up to three in others
+    cfg = {n: (1 if j % 2 else 3) for j, n in enumerate(names)}
+    freed, loaded = ck.apply_compression_config(str(tmp_path), linears, cfg)
+    assert freed == sum(linears[n].memory_per_bit() for n in names if cfg[n] == 1)
+    assert loaded == sum(linears[n].memory_per_bit() for n in names if cfg[n] == 3)
+    for n in names:
+        mod = linears[n]
+        assert mod.w_bit == cfg[n] and mod.u.shape[0] == cfg[n] and mod.qweight.shape[0] == cfg[n] and mod.vt.shape[0] == cfg[n]
+        _, L, proj = n.split(".", 2)
+        for i in range(cfg[n]):
+            assert torch.equal(mod.qweight[i], tensors[f"model.layers.{L}.{proj}.qweight_{i}"])
+            assert torch.equal(mod.u[i], tensors[f"model.layers.{L}.{proj}.u_{i}"])
+    # a counter-only change (the reference's set_bit) followed by growth: surplus is dropped first
+    m = linears[names[0]]
+    m.set_bit(1)
+    assert m.u.shape[0] == 3
+    ck.apply_compression_config(str(tmp_path), linears, {**cfg, names[0]: 2})
+    assert m.w_bit == 2 and m.u.shape[0] == 2 and torch.equal(m.vt[1], tensors["model.layers.0.self_attn.q_proj.vt_1"])
+    with pytest.raises(KeyError):
+        ck.apply_compression_config(str(tmp_path), linears, {**cfg, names[0]: 4})
+    with pytest.raises(RuntimeError):
+        m.set_bit(1)
+        m.append_blocks(m.qweight[:1], m.u[:1], m.vt[:1])
+    # values: the level-0 forward needs per-block buffers, so compare through the stacked tensors
+    for n in names[:2]:
+        mod = linears[n]
+        mod.set_bit(mod.u.shape[0])
+        w = sum(bo.compose_weight(mod.qweight[i].numpy(), mod.u[i].numpy().astype(np.float32), mod.vt[i].numpy().astype(np.float32),
+                                  weight_shape=(mod.out_features, mod.in_features)) for i in range(mod.w_bit))
+        y = x[n].numpy().astype(np.float64) @ w.astype(np.float64).T + (0 if mod.bias is None else mod.bias.numpy().astype(np.float64))
+        ref = dense_out(n, mod.w_bit)
+        assert np.abs(y - ref).max() <= 1e-3 * max(np.abs(ref).max(), 1e-6)

@@ -268,3 +268,36 @@ def test_non_contiguous_input_is_handled():
     wide[:, ::2] = x
     y = IU.bitstack_forward_hip(q, u, vt, wide[:, ::2])
     assert torch.equal(y, IU.bitstack_forward_hip(q, u, vt, x))
+
+
+# ------------------------------------------------------------- decomposition on the GPU
+def test_decompose_on_gpu_matches_oracle():
+    """from_linear on a HIP tensor (BitStackLinear.py:49-86): SVD through torch (rocSOLVER), signs
+    packed by the HIP kernel.  Factors are only defined up to a joint sign per rank, so products
+    are compared; the first block's signs are those of the weight itself and must match bit for bit."""
+    print("decompose on gpu", flush=True)
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(192, 256, bias=True)
+    with torch.no_grad():
+        lin.weight.mul_(0.5)
+    lin = lin.half()                      # the reference decomposes fp16 checkpoints
+    w = lin.weight.detach().float().numpy().copy()
+    q_ref, u_ref, vt_ref, norms = O.decompose_weight(w, 3, 8)
+    with torch.no_grad():                 # as the reference's decompose() (bitstack/utils/decompose.py:7)
+        mod = BitStackLinear.from_linear(lin.to(dev()), w_bit=3, k=8, bias=True, fused_level=5, name="t")
+    assert mod.qweight_0.is_cuda and mod.u_0.dtype == torch.float16
+    assert np.array_equal(mod.qweight_0.cpu().numpy(), q_ref[0])
+    res = w.astype(np.float64)
+    for i in range(3):
+        p_gpu = getattr(mod, f"u_{i}").double().cpu().numpy() @ getattr(mod, f"vt_{i}").double().cpu().numpy()
+        p_ref = u_ref[i].astype(np.float64) @ vt_ref[i].astype(np.float64)
+        assert np.abs(p_gpu - p_ref).max() <= 2e-3 * np.abs(p_ref).max(), i
+        s = O.unpack_sign(getattr(mod, f"qweight_{i}").cpu().numpy(), w.shape).astype(np.float64)
+        res = res - s * p_gpu
+        # the residual shrinks like the oracle's (Eckart-Young step by step)
+        assert abs(np.linalg.norm(res) - norms[i + 1]) <= 2e-2 * norms[i + 1], i
+    mod.stack_blocks()
+    x = torch.randn(2, 192, generator=torch.Generator().manual_seed(1)).half()
+    y = mod(x.to(dev())).float().cpu().numpy()
+    want = x.double().numpy() @ (w.astype(np.float64) - res).T + lin.bias.detach().double().cpu().numpy()
+    assert_close(y, want, "decomposed layer forward vs fp64")
