@@ -155,7 +155,7 @@ struct GemvGroup {
 };
 
 template <int T, int WAVES, int R>
-__global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? 2 : 1))) void gemv_kernel(
+__global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? (WAVES == 8 && R == 2 ? 4 : 2) : 1))) void gemv_kernel(
     const GemvGroup grp, const half_t *__restrict__ x, int N, int K, int n_chunks) {
     constexpr int RW = WAVES * R * 16;          // rows per workgroup
     constexpr int COMBOS = 8 / WAVES;           // (jb, pg) producer combos per wave
@@ -522,11 +522,16 @@ Plan make_plan(const int *I, const int *M, int n, int N, int T) {
     Plan p;
     p.n = n;
     p.n_chunks = N / CH;
-    // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU
-    const int cand[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
+    // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU.
+    // Three or four tokens need more than the 128 registers a lane has with two 8-wave
+    // workgroups of four row tiles per CU: there the tall candidate is 8 waves x 2 tiles
+    // (one workgroup per CU, two waves per SIMD to overlap sign decode and MFMA).
+    const int cand1[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
+    const int cand3[4][3] = {{8, 2, 1}, {4, 4, 1}, {4, 2, 1}, {4, 1, 1}};
+    const int cand2[4][3] = {{8, 2, 2}, {4, 4, 2}, {4, 2, 2}, {4, 1, 2}};
+    const int (*cand)[3] = T > 2 ? cand3 : T == 2 ? cand2 : cand1;
     int pick = 3;
-    // three or four tokens need more than the 256 registers an 8-wave workgroup can have
-    for (int k = (T > 2 ? 1 : 0); k < 4; k++) {
+    for (int k = 0; k < 4; k++) {
         const int rw = cand[k][0] * cand[k][1] * 16;
         bool tall = true;
         int64_t units = 0;
@@ -596,8 +601,8 @@ int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int 
 template <int T>
 int launch_T(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     if (p.waves == 8) {
-        if constexpr (T <= 2) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
-        else return BS_ERR_SHAPE;     // the planner never pairs 8 waves with more than two tokens
+        if constexpr (T == 1) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
+        else return launch_one<T, 8, 2>(p, grp, x, N, K, s);
     }
     if (p.R == 4) return launch_one<T, 4, 4>(p, grp, x, N, K, s);
     if (p.R == 2) return launch_one<T, 4, 2>(p, grp, x, N, K, s);
