@@ -20,8 +20,9 @@
 //     j = 9..4 (mantissa)  {4,6} {8,10} {16,18} {32,34} {64,66} {128,130}
 // Then s = v - mid_j, and   sum_n s_n z_n = sum_n v_n z_n - sum_n mid_n z_n.
 // The first sum is what the MFMAs accumulate; the second does not depend on
-// the row and is accumulated by wave 0 with one extra MFMA per step against a
-// constant operand.  All codes are exact in fp16 and every product is exact
+// the row; the waves of a workgroup share it out (16 / WAVES steps each, one extra
+// MFMA per step against a constant operand) and exchange their shares through LDS
+// when a row is flushed.  All codes are exact in fp16 and every product is exact
 // in fp32, so the only extra error is fp32 accumulation of terms up to 129x
 // larger than z (about 1e-5 relative, far below the fp16 rounding of y).
 // Bit positions 10..13 and 0..3 have no such code (or a badly conditioned
@@ -33,9 +34,11 @@
 // ---- work split ------------------------------------------------------------
 // The matrix stack is cut into UNITS: (block i, row tile of WAVES*R*16 rows,
 // 512-column chunk), ordered with the chunk fastest.  The grid is persistent:
-// about two workgroups per CU, each owning one contiguous range of units of
-// equal length, so the load is balanced for any shape and each workgroup pays
-// its pipeline fill once.  Per unit every lane reads its 16 bytes of signs
+// about two workgroups per CU (one for three or four tokens), each owning one
+// contiguous range of units of equal length, so the load is balanced for any
+// shape and each workgroup pays its pipeline fill once.  Up to four matrices that
+// read the same x share a launch: the grid is cut into one run of workgroups per
+// matrix.  Per unit every lane reads its 16 bytes of signs
 // (128 columns of one row) with one 128-bit load per row tile, one unit ahead
 // of use; Z for unit u+1 is produced by all threads (vt and x loads issued
 // before the MFMA loop of unit u, finished after it) into the other half of a
@@ -43,8 +46,8 @@
 // unit.  Accumulators are flushed whenever the range crosses into another
 // (block, row tile): scaled by u, reduced over ranks, written as a partial
 // row sum to scratch [I, KMAX, T, M] (fp32).  A second kernel adds the
-// partials of a row in a fixed order, adds the bias and rounds to fp16:
-// deterministic, no atomics.  Workgroups with neighbouring ranges - which read
+// partials of a row in a fixed order, adds the bias, rounds to fp16 and applies
+// the epilogue (none, + residual, silu(a) * b): deterministic, no atomics.  Workgroups with neighbouring ranges - which read
 // the same slices of vt - sit on the same XCD (and share its L2).
 #include "common.h"
 
