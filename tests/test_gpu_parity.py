@@ -301,3 +301,33 @@ def test_decompose_on_gpu_matches_oracle():
     y = mod(x.to(dev())).float().cpu().numpy()
     want = x.double().numpy() @ (w.astype(np.float64) - res).T + lin.bias.detach().double().cpu().numpy()
     assert_close(y, want, "decomposed layer forward vs fp64")
+
+
+# ------------------------------------------------------------- seeded random shapes
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        kind = rng.integers(0, 4)
+        if kind == 0:      # decode kernel shapes: N a multiple of 512, any M
+            N = 512 * int(rng.integers(1, 9)); M = int(rng.integers(1, 700)); T = int(rng.integers(1, 9))
+        elif kind == 1:    # tiled rebuild + GEMM: N a multiple of 128, more tokens
+            N = 128 * int(rng.integers(1, 12)); M = int(rng.integers(1, 500)); T = int(rng.integers(9, 200))
+        elif kind == 2:    # N only a multiple of 8: generic rebuild, k-tail GEMM / skinny
+            N = 8 * int(rng.integers(1, 90)); M = int(rng.integers(1, 300)); T = int(rng.integers(1, 70))
+        else:              # tall matrices through the 8-wave decode kernels
+            N = 512 * int(rng.integers(1, 4)); M = 512 * int(rng.integers(1, 5)) + int(rng.integers(0, 3)) * 7; T = int(rng.integers(1, 5))
+        cases.append((int(rng.integers(1, 7)), M, N, T, int(rng.choice([16, 16, 16, 8, 3]))))
+    return cases
+
+
+@pytest.mark.parametrize("I,M,N,T,K", _random_cases(48, 20240607))
+def test_forward_random_shapes(I, M, N, T, K):
+    print(f"forward random I={I} M={M} N={N} T={T} K={K}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=M + N + T, signed_factors=True)
+    bias = (torch.randn(M, generator=torch.Generator().manual_seed(I)) * 0.05).half() if (M + T) % 2 else None
+    exact, _ = oracle_refs(q, u, vt, x, bias)
+    y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev()),
+                                None if bias is None else bias.to(dev())).cpu().numpy()
+    assert y.shape == (T, M)
+    assert_close(y, exact, "vs fp64")
