@@ -81,3 +81,12 @@ def unpack_sign(packed, original_shape):
     if packed.is_cuda:
         return unpack_sign_hip(packed, original_shape)
     return _unpack_sign_torch(packed, original_shape)
+
+
+def unpack_sign_v2(packed, original_shape):
+    """Same mapping and the same dtype check as the reference's second variant
+    (bitstack/utils/pack_utils.py:50-82, a cached-mask rewrite of unpack_sign)."""
+    if packed.dtype != torch.uint8:
+        raise ValueError(f"Expected packed tensor of dtype torch.uint8, but got {packed.dtype}")
+    return unpack_sign(packed, torch.Size(original_shape))
+

@@ -135,3 +135,15 @@ def test_algorithmic_bytes_closed_form():
     assert algorithmic_bytes(1, 4096, 4096, 1) == 2_097_152 + 262_144 + 16_384
     assert round(algorithmic_bytes(8, 4096, 4096, 1) / 1e6, 3) == 18.891
     assert round(algorithmic_bytes(16, 4096, 14336, 1) / 1e6, 3) == 126.915
+
+
+def test_unpack_sign_v2_is_the_same_mapping_with_a_dtype_check():
+    from bitstack_amd.utils.pack_utils import unpack_sign_v2
+    rng = np.random.default_rng(3)
+    packed = torch.from_numpy(rng.integers(0, 256, size=13, dtype=np.uint8))
+    for shape in [(100,), (4, 26), (13, 8)]:
+        got = unpack_sign_v2(packed, torch.Size(shape)).numpy()
+        want = np.unpackbits(packed.numpy(), bitorder="big")[: int(np.prod(shape))].astype(np.int8).reshape(shape) * 2 - 1
+        assert np.array_equal(got, want)
+    with pytest.raises(ValueError):
+        unpack_sign_v2(packed.to(torch.int16), torch.Size((8,)))
