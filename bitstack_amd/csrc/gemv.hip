@@ -439,25 +439,27 @@ struct RedGroup {
 // Sum of the partials of output m of one matrix that this thread's slice covers.
 // The (block, slot) pairs are numbered i * kmax + k and slice ks takes every
 // RED_SL-th of them, four at a time: slots that are not live (k beyond the number of
-// workgroups that touched this row tile of block i) are loaded from a live address
-// and masked, so the four loads never wait for one another or for the counts.
-__device__ __forceinline__ float slice_sum_any(const RedMat &r, int T, int t, int m, int rt, int n_chunks, int ks) {
+// workgroups that touched this row tile of block i, `nks[i]`, worked out once per
+// workgroup) are loaded all the same (the slots exist in the workspace) and masked, so
+// the loads of a batch never wait for one another.  (i, k) advance incrementally: no
+// division in the loop.
+__device__ __forceinline__ float slice_sum_any(const RedMat &r, int T, int t, int m, int ks, const int *nks) {
     const int total = r.I * r.kmax;
     const int64_t stride = (int64_t)T * r.M;
     const float *base = r.part + (int64_t)t * r.M + m;
     float acc = 0.f;
+    int i = ks / r.kmax, k = ks - i * r.kmax;                  // slot ks
     for (int s0 = ks; s0 < total; s0 += 4 * RED_SL) {
         float v[4];
         bool ok[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int s = s0 + j * RED_SL;
-            const int sc = s < total ? s : ks;                 // slot ks exists whenever the loop runs
-            const int i = sc / r.kmax, k = sc - i * r.kmax;
-            const int first = (i * r.row_tiles + rt) * n_chunks;
-            const int nk = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
-            ok[j] = s < total && k < nk;
-            v[j] = base[(int64_t)(i * r.kmax + (k < nk ? k : 0)) * stride];
+            const bool in = s0 + j * RED_SL < total;
+            const int ic = in ? i : 0, kc = in ? k : 0;
+            ok[j] = in && kc < nks[ic];
+            v[j] = base[(int64_t)(ic * r.kmax + kc) * stride];
+            k += RED_SL;
+            while (k >= r.kmax) { k -= r.kmax; i++; }
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) acc += ok[j] ? v[j] : 0.f;
@@ -465,10 +467,19 @@ __device__ __forceinline__ float slice_sum_any(const RedMat &r, int T, int t, in
     return acc;
 }
 
+// nks[i] = workgroups whose unit range touched (block i, row tile rt) of this matrix
+__device__ __forceinline__ void count_partials(const RedMat &r, int rt, int n_chunks, int *nks) {
+    for (int i = threadIdx.x; i < r.I; i += RED_OUT * RED_SL) {
+        const int first = (i * r.row_tiles + rt) * n_chunks;
+        nks[i] = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
+    }
+}
+
 __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy,
     int rows_per_tile, int n_chunks) {
     __shared__ float red[2][RED_SL][RED_OUT];
+    __shared__ int nks[2][RED_MAXBLOCKS];
     const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
     int j = 0;
     if (grp.mode != EPI_SWIGLU) {
@@ -484,14 +495,17 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
     const bool live = m < r.M;
     const bool two = grp.mode == EPI_SWIGLU;
+    count_partials(r, rt, n_chunks, nks[0]);
+    if (two) count_partials(grp.m[1], rt, n_chunks, nks[1]);
     // residual and bias do not depend on the sums: fetch them before the reduction
     float extra = 0.f, res = 0.f;
     if (ks == 0 && live) {
         if (r.bias) extra = (float)r.bias[m];
         if (grp.mode == EPI_RESIDUAL) res = (float)residual[(int64_t)t * ldy + r.y_off + m];
     }
-    red[0][ks][lo] = live ? slice_sum_any(r, T, t, m, rt, n_chunks, ks) : 0.f;
-    if (two) red[1][ks][lo] = live ? slice_sum_any(grp.m[1], T, t, m, rt, n_chunks, ks) : 0.f;
+    __syncthreads();
+    red[0][ks][lo] = live ? slice_sum_any(r, T, t, m, ks, nks[0]) : 0.f;
+    if (two) red[1][ks][lo] = live ? slice_sum_any(grp.m[1], T, t, m, ks, nks[1]) : 0.f;
     __syncthreads();
     if (ks != 0 || !live) return;
     float s0 = extra;
