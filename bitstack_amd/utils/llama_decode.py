@@ -112,20 +112,25 @@ class SyntheticLlamaDecoder:
                   them, all from the library."""
 
     def __init__(self, shape: LlamaShape, config: dict, max_len: int, device, seed=0, batch=1):
-        self.s, self.dev, self.max_len, self.batch = shape, torch.device(device), max_len, batch
-        g = torch.Generator(device=self.dev).manual_seed(seed)
+        dev = torch.device(device)
+        g = torch.Generator(device=dev).manual_seed(seed)
         h = shape.hidden
-        self.embed = (torch.randn(shape.vocab, h, device=self.dev, generator=g) * 0.02).half()
-        self.lm_head = (torch.randn(shape.vocab, h, device=self.dev, generator=g) * 0.02).half()
-        self.norm_w = torch.ones(shape.layers, 2, h, device=self.dev, dtype=torch.float16)
-        self.final_norm = torch.ones(h, device=self.dev, dtype=torch.float16)
-        self.lin = []
+        embed = (torch.randn(shape.vocab, h, device=dev, generator=g) * 0.02).half()
+        lm_head = (torch.randn(shape.vocab, h, device=dev, generator=g) * 0.02).half()
+        norm_w = torch.ones(shape.layers, 2, h, device=dev, dtype=torch.float16)
+        final_norm = torch.ones(h, device=dev, dtype=torch.float16)
+        lin = []
         for L in range(shape.layers):
             row = {}
             for p in PROJ:
                 m, n = shape.proj_shape(p)
-                row[p] = _synthetic_bitstack(m, n, config[f"layer.{L}.{p}"], shape.k, self.dev, g, f"layer.{L}.{p}")
-            self.lin.append(row)
+                row[p] = _synthetic_bitstack(m, n, config[f"layer.{L}.{p}"], shape.k, dev, g, f"layer.{L}.{p}")
+            lin.append(row)
+        self._setup(shape, lin, embed, lm_head, norm_w, final_norm, max_len, dev, batch)
+
+    def _setup(self, shape, lin, embed, lm_head, norm_w, final_norm, max_len, dev, batch):
+        self.s, self.dev, self.max_len, self.batch = shape, dev, max_len, batch
+        self.lin, self.embed, self.lm_head, self.norm_w, self.final_norm = lin, embed, lm_head, norm_w, final_norm
         d = shape.head_dim
         self.kcache = torch.zeros(shape.layers, batch, shape.kv_heads, max_len, d, device=self.dev, dtype=torch.float16)
         self.vcache = torch.zeros_like(self.kcache)
@@ -137,6 +142,59 @@ class SyntheticLlamaDecoder:
         self.span = torch.arange(max_len, device=self.dev)
         self.logits = None
         self._groups = None
+
+    @classmethod
+    def from_checkpoint(cls, path, max_len, device, compression_config=None, niter=None, max_memory_MB=None, batch=1):
+        """A decoder over a compressed checkpoint in the reference's layout on local disk
+        (bitstack_amd/utils/checkpoint.py): `config.json` supplies the Llama dimensions
+        (Hugging Face keys), `compression_config.json` + max_memory_MB pick the blocks per
+        layer as the reference's --max_memory_MB does (bitstack/main.py:85-91), or pass a
+        compression_config / niter directly.  Token ids in, token ids out: no tokenizer."""
+        import json
+        import os
+        from bitstack_amd.utils import checkpoint as ck
+        with open(os.path.join(path, "config.json"), "r") as f:
+            hf = json.load(f)
+        rope = hf.get("rope_theta") or (hf.get("rope_parameters") or {}).get("rope_theta", 10000.0)
+        shape = LlamaShape(layers=hf["num_hidden_layers"], hidden=hf["hidden_size"], intermediate=hf["intermediate_size"],
+                           heads=hf["num_attention_heads"], kv_heads=hf.get("num_key_value_heads", hf["num_attention_heads"]),
+                           vocab=hf["vocab_size"], rope_theta=float(rope), rms_eps=float(hf.get("rms_norm_eps", 1e-5)))
+        if hf.get("head_dim", shape.head_dim) != shape.head_dim:
+            raise ValueError("head_dim other than hidden_size / num_attention_heads is not supported")
+        if max_memory_MB is not None:
+            compression_config = ck.retrieve_compression_config(ck.read_compression_configs(path), max_memory_MB)
+        dev = torch.device(device)
+        linears, other = ck.load_bitstack_checkpoint(path, compression_config=compression_config, niter=niter,
+                                                     device=dev, fused_level=5)
+        lin = [{p: linears[f"layer.{L}.{p}"] for p in PROJ} for L in range(shape.layers)]
+        shape.k = lin[0][PROJ[0]].k
+        f16 = lambda t: t.to(dev, torch.float16).contiguous()
+        norm_w = torch.stack([torch.stack([f16(other[f"model.layers.{L}.input_layernorm.weight"]),
+                                           f16(other[f"model.layers.{L}.post_attention_layernorm.weight"])])
+                              for L in range(shape.layers)])
+        embed = f16(other["model.embed_tokens.weight"])
+        lm_head = f16(other["lm_head.weight"]) if "lm_head.weight" in other else embed      # tied embeddings
+        self = cls.__new__(cls)
+        self._setup(shape, lin, embed, lm_head, norm_w, f16(other["model.norm.weight"]), max_len, dev, batch)
+        return self
+
+    def save_checkpoint(self, path, compression_configs=None, max_shard_bytes=None):
+        """Writes this decoder in the same layout (config.json included)."""
+        import json
+        import os
+        from bitstack_amd.utils import checkpoint as ck
+        s = self.s
+        linears = {f"layer.{L}.{p}": self.lin[L][p] for L in range(s.layers) for p in PROJ}
+        other = {"model.embed_tokens.weight": self.embed, "lm_head.weight": self.lm_head, "model.norm.weight": self.final_norm}
+        for L in range(s.layers):
+            other[f"model.layers.{L}.input_layernorm.weight"] = self.norm_w[L, 0]
+            other[f"model.layers.{L}.post_attention_layernorm.weight"] = self.norm_w[L, 1]
+        ck.save_bitstack_checkpoint(path, linears, other, compression_configs, max_shard_bytes)
+        with open(os.path.join(path, "config.json"), "w") as f:
+            json.dump({"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": s.layers,
+                       "hidden_size": s.hidden, "intermediate_size": s.intermediate, "num_attention_heads": s.heads,
+                       "num_key_value_heads": s.kv_heads, "vocab_size": s.vocab, "rope_theta": s.rope_theta,
+                       "rms_norm_eps": s.rms_eps, "tie_word_embeddings": False}, f)
 
     def weight_bytes(self):
         b = self.embed.numel() * 2 + self.lm_head.numel() * 2

@@ -231,3 +231,28 @@ def test_fused_step_replays_in_a_graph():
         torch.cuda.synchronize()
         assert torch.equal(m.logits, ref.logits), step
         assert torch.equal(m.token, ref.token) and int(m.pos) == step + 1
+
+
+def test_decoder_round_trips_through_a_checkpoint(tmp_path):
+    """save_checkpoint -> from_checkpoint (reference layout: sharded safetensors, config.json,
+    compression_config.json) gives the same logits; a smaller memory budget loads fewer blocks."""
+    cfg = {k: 3 for k in small_config()}
+    a = SyntheticLlamaDecoder(SMALL, cfg, 16, dev(), seed=6)
+    with torch.no_grad():
+        a.norm_w.copy_(1 + 0.1 * torch.randn(a.norm_w.shape, device=dev(), generator=torch.Generator(device=dev()).manual_seed(1)))
+    per_block = sum(m.memory_per_bit() for row in a.lin for m in row.values())
+    dense = 2 * (a.embed.numel() + a.lm_head.numel())
+    configs = [{"memory": dense + b * per_block, "layers": {k: b for k in cfg}} for b in (1, 2, 3)]
+    a.save_checkpoint(str(tmp_path), compression_configs=configs, max_shard_bytes=200_000)
+    full_mb = (dense + 3 * per_block) / 1024 ** 2 + 0.01
+    b = SyntheticLlamaDecoder.from_checkpoint(str(tmp_path), 16, dev(), max_memory_MB=full_mb)
+    small = SyntheticLlamaDecoder.from_checkpoint(str(tmp_path), 16, dev(), max_memory_MB=(dense + 2 * per_block) / 1024 ** 2 + 0.01)
+    assert all(m.w_bit == 3 for row in b.lin for m in row.values())
+    assert all(m.w_bit == 2 and m.u.shape[0] == 2 for row in small.lin for m in row.values())
+    for tok in (5, 9, 200, 31):
+        for m in (a, b, small):
+            m.token.fill_(tok)
+            m.step_fused()
+        assert torch.equal(a.logits, b.logits)
+        assert not torch.equal(a.logits, small.logits)
+    assert torch.equal(a.token, b.token)
