@@ -541,10 +541,11 @@ Plan make_plan(const int *I, const int *M, int n, int N, int T) {
     p.n_chunks = N / CH;
     // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU.
     // Three or four tokens need more than the 128 registers a lane has with two 8-wave
-    // workgroups of four row tiles per CU: there the tall candidate is 8 waves x 2 tiles
-    // (one workgroup per CU, two waves per SIMD to overlap sign decode and MFMA).
+    // workgroups per CU: there it is one workgroup of 8 waves per CU (two waves per SIMD
+    // to overlap sign decode and MFMA), four row tiles per wave (each Z fragment read
+    // from LDS feeds four MFMAs per token) or two when the layer has too few units.
     const int cand1[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
-    const int cand3[4][3] = {{8, 2, 1}, {4, 4, 1}, {4, 2, 1}, {4, 1, 1}};
+    const int cand3[4][3] = {{8, 4, 1}, {8, 2, 1}, {4, 2, 1}, {4, 1, 1}};
     const int cand2[4][3] = {{8, 2, 2}, {4, 4, 2}, {4, 2, 2}, {4, 1, 2}};
     const int (*cand)[3] = T > 2 ? cand3 : T == 2 ? cand2 : cand1;
     int pick = 3;
@@ -618,8 +619,10 @@ int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int 
 template <int T>
 int launch_T(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     if (p.waves == 8) {
-        if constexpr (T == 1) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
-        else return launch_one<T, 8, 2>(p, grp, x, N, K, s);
+        if constexpr (T == 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
+        else if (p.R == 4) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
+        else if constexpr (T > 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
+        else return BS_ERR_SHAPE;
     }
     if (p.R == 4) return launch_one<T, 4, 4>(p, grp, x, N, K, s);
     if (p.R == 2) return launch_one<T, 4, 2>(p, grp, x, N, K, s);
