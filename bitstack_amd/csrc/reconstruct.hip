@@ -5,12 +5,13 @@
 // Tiled kernel.  A workgroup owns a strip of 128 columns and a range of rows.
 // It first stages the strip's slice of vt for ALL blocks in LDS, transposed to
 // [block][column][rank] (vt is stored rank-major, the MFMA wants the rank
-// index contiguous per lane; column stride 20 halves keeps the 8-byte fragment
-// reads aligned and off each other's banks), then walks its rows 16 per wave at a time with
+// index contiguous per lane; 16 halves per column plus 4 after every 8 columns keeps
+// the 8-byte fragment reads aligned and off each other's banks), then walks its rows 16 per wave at a time with
 // no further barrier.  Per block the rank-k product of a 16 x 16 patch is one
 // v_mfma_f32_16x16x16_f16 computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
-// so that a lane ends up with four consecutive columns of one row - exactly
-// one nibble of that row's packed sign byte.  The sign is moved to bit 31,
+// so that a lane ends up with four consecutive columns of one row - one nibble
+// of that row's packed sign byte - and, over a pair of patches, with a whole byte
+// (eight consecutive columns, one 16-byte store).  The sign is moved to bit 31,
 // merged into the constant 1.0f and applied with one FMA.  Signs and u of the
 // next block are loaded while the current block is multiplied.
 #include "common.h"
@@ -18,15 +19,17 @@
 namespace {
 
 constexpr int RT_COLS = 128;   // columns per workgroup strip
-constexpr int VSTRIDE = 20;    // halves between consecutive columns in LDS (8-byte aligned fragments)
-constexpr int RT_MAXB = 30;    // most blocks whose vt strip fits in LDS (30 x 5 KB)
+constexpr int VSTRIDE = 16;    // halves per column in LDS: the 16 ranks, contiguous
+constexpr int VGROUP_PAD = 4;  // extra halves after every 8 columns (keeps the fragment reads off each other's banks)
+constexpr int VBLOCK = RT_COLS * VSTRIDE + (RT_COLS / 8) * VGROUP_PAD;   // halves per block in LDS
+constexpr int RT_MAXB = 36;    // most blocks whose vt strip fits in LDS (36 x 4.1 KB)
 
 template <bool PACKED>
 __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
     const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
     const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
     int I, int M, int N, int K, int rows_per_wg) {
-    extern __shared__ __attribute__((aligned(16))) half_t vl[];   // [I][RT_COLS][VSTRIDE]
+    extern __shared__ __attribute__((aligned(16))) half_t vl[];   // [I][VBLOCK]: column c of a block at c * 16 + (c / 8) * 4
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lm = lane & 15, g = lane >> 4;
@@ -51,17 +54,42 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
 
     // staging role: rank index fastest across lanes, 16 pieces of 8 columns
     const int sr = tid & 15, sp = tid >> 4;
-    // shift that brings this lane's first column of an even 16-column patch to bit 31
-    const int sh_even = 24 - 8 * (g >> 1) + 4 * (g & 1);
+    // Patches come in pairs: of a 32-column group, patch 2q takes columns 8g'..8g'+3 and patch
+    // 2q+1 columns 8g'+4..8g'+7 (g' = 0..3), so that a lane (row lm, group g) ends up with EIGHT
+    // consecutive columns of its row - one byte of the packed signs, one 16-byte store.
+    // Shift that brings the lane's byte of a sign word to the top (first column at bit 31):
+    const int sh_byte = 24 - 8 * g;
+    // this lane's A-fragment column within a 32-column group (n-index lm of either patch, less 4 * (s & 1))
+    const int acol = 8 * (lm >> 2) + (lm & 3);
+    const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
 
     {
         const int i0 = 0, ib = I;
+        // u rows and sign words of one (row step, block); requested one block ahead, also
+        // across the end of a row step (first block of the next 16 rows), and issued for
+        // the very first block before the vt strip is staged
+        auto load_block = [&](int i, int row, half4_t &b, uint4_t &sw) {
+            const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+            if (K == 16) {
+                b = *reinterpret_cast<const half4_t *>(up);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
+            }
+            if (PACKED) {
+                sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
+            }
+        };
+        half4_t b_cur, b_nxt;
+        uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
+        if (row_begin + wave * 16 < row_end) load_block(i0, min(row_begin + wave * 16 + lm, M - 1), b_cur, sw_cur);
+
         for (int i = 0; i < ib; i++) {
             half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
             if (sr < K)
                 v = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
 #pragma unroll
-            for (int e = 0; e < 8; e++) vl[(i * RT_COLS + 8 * sp + e) * VSTRIDE + sr] = v[e];
+            for (int e = 0; e < 8; e++) vl[i * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[e];
         }
         __syncthreads();
 
@@ -72,33 +100,18 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
 #pragma unroll
             for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
-            auto load_block = [&](int i, half4_t &b, uint4_t &sw) {
-                const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
-                if (K == 16) {
-                    b = *reinterpret_cast<const half4_t *>(up);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
-                }
-                if (PACKED) {
-                    sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
-                }
-            };
-
-            half4_t b_cur, b_nxt;
-            uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
-            load_block(i0, b_cur, sw_cur);
             for (int i = 0; i < ib; i++) {
-                if (i + 1 < ib) load_block(i0 + i + 1, b_nxt, sw_nxt);
+                if (i + 1 < ib) load_block(i0 + i + 1, row, b_nxt, sw_nxt);
+                else if (m0 + 64 < row_end) load_block(i0, min(m0 + 64 + lm, M - 1), b_nxt, sw_nxt);
                 const uint4_t swc = ~sw_cur;     // bit 1 means +1: make it a clear IEEE sign bit
-                const half_t *vb = vl + (i * RT_COLS) * VSTRIDE;
+                const half_t *vb = vl + i * VBLOCK + aoff;
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
-                    const half_t *ap = vb + (16 * s + lm) * VSTRIDE + 4 * g;
+                    const half_t *ap = vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD;
                     const half4_t a = *reinterpret_cast<const half4_t *>(ap);
                     float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     if (PACKED) {
-                        uint32_t t = swc[s >> 1] << (sh_even - 16 * (s & 1));
+                        uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
@@ -106,7 +119,7 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                         }
                     } else {
                         uint32_t t = *reinterpret_cast<const uint32_t *>(
-                            sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 16 * s + 4 * g);
+                            sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 32 * (s >> 1) + 8 * g + 4 * (s & 1));
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
@@ -119,11 +132,12 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
             }
 
             if (m0 + lm < M) {
-                half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 4 * g;
+                half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 8 * g;
 #pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    half4_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-                    *reinterpret_cast<half4_t *>(wp + 16 * s) = o;
+                for (int s = 0; s < 8; s += 2) {
+                    half8_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3],
+                                 (half_t)acc[s + 1][0], (half_t)acc[s + 1][1], (half_t)acc[s + 1][2], (half_t)acc[s + 1][3]};
+                    *reinterpret_cast<half8_t *>(wp + 16 * s) = o;      // 32 columns per pair of patches
                 }
             }
         }
@@ -163,14 +177,14 @@ __global__ __launch_bounds__(256) void reconstruct_generic_kernel(
 template <bool PACKED>
 int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *u, const half_t *vt,
                        half_t *w, int I, int M, int N, int K, hipStream_t s) {
-    const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && bs_aligned(vt, 16) && bs_aligned(w, 8) &&
+    const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && bs_aligned(vt, 16) && bs_aligned(w, 16) &&
                        bs_aligned(u, 8) && (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
     if (tiled) {
         // One wave of workgroups: as many row groups as the resident slots allow (LDS decides
         // how many workgroups a CU holds), so that no second, partial wave trails behind.
         // Every workgroup re-stages its vt strip, so rows per workgroup stay a multiple of 64.
         const int strips = N / RT_COLS, strips8 = (int)bs_cdiv(strips, 8) * 8;
-        const size_t lds_need = (size_t)I * RT_COLS * VSTRIDE * sizeof(half_t);
+        const size_t lds_need = (size_t)I * VBLOCK * sizeof(half_t);
         int per_cu = (int)((160 * 1024) / lds_need);
         if (per_cu > 8) per_cu = 8;
         if (per_cu < 1) per_cu = 1;
@@ -178,7 +192,7 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
         if (row_groups < 1) row_groups = 1;
         int rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
         row_groups = (int)bs_cdiv(M, rows_per_wg);
-        const size_t lds = (size_t)I * RT_COLS * VSTRIDE * sizeof(half_t);
+        const size_t lds = lds_need;
         static size_t raised = 0;
         if (lds > 64 * 1024 && lds > raised) {
             BS_HIP_TRY(hipFuncSetAttribute((const void *)reconstruct_tile_kernel<PACKED>,
