@@ -94,9 +94,9 @@ extern "C" int64_t bs_forward_group_workspace_bytes(const bs_matrix *mats, int n
     return b > 0 ? round_up(b, 256) : (int64_t)BS_ERR_SHAPE;
 }
 
-extern "C" int bs_forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, int T,
-                                int epilogue, const void *residual, void *y,
-                                void *workspace, int64_t workspace_bytes, void *stream) {
+static int forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, int T,
+                         int epilogue, const void *residual, void *y, int input_rms, float eps,
+                         void *workspace, int64_t workspace_bytes, void *stream) {
     int st = group_dims(mats, n, N, K, T);
     if (st != BS_OK) return st;
     if (epilogue != BS_EPI_NONE && epilogue != BS_EPI_RESIDUAL && epilogue != BS_EPI_SWIGLU) return BS_ERR_SHAPE;
@@ -121,8 +121,21 @@ extern "C" int bs_forward_group(const bs_matrix *mats, int n, int N, int K, cons
     if (need < 0) return (int)need;
     if (!workspace || workspace_bytes < need || !bs_aligned(workspace, 256)) return BS_ERR_WORKSPACE;
     return bs_launch_gemv_group(n, packed, u, vt, bias, I, M, N, K, (const half_t *)x, T, epilogue,
-                                (const half_t *)residual, (half_t *)y, workspace, workspace_bytes,
+                                (const half_t *)residual, (half_t *)y, input_rms, eps, workspace, workspace_bytes,
                                 (hipStream_t)stream);
+}
+
+extern "C" int bs_forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, int T,
+                                int epilogue, const void *residual, void *y,
+                                void *workspace, int64_t workspace_bytes, void *stream) {
+    return forward_group(mats, n, N, K, x, T, epilogue, residual, y, 0, 0.f, workspace, workspace_bytes, stream);
+}
+
+extern "C" int bs_forward_group_rms(const bs_matrix *mats, int n, int N, int K, const void *x, int T, float eps,
+                                    int epilogue, const void *residual, void *y,
+                                    void *workspace, int64_t workspace_bytes, void *stream) {
+    if (!(eps >= 0.f)) return BS_ERR_SHAPE;
+    return forward_group(mats, n, N, K, x, T, epilogue, residual, y, 1, eps, workspace, workspace_bytes, stream);
 }
 
 extern "C" int bs_rmsnorm_f16(const void *x, const void *weight, void *y, int T, int H, float eps, void *stream) {

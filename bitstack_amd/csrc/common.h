@@ -48,8 +48,8 @@ enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, int K, int T);
 int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
                          const half_t *const *bias, const int *I, const int *M, int N, int K, const half_t *x, int T,
-                         int mode, const half_t *residual, half_t *y, void *workspace, int64_t workspace_bytes,
-                         hipStream_t s);
+                         int mode, const half_t *residual, half_t *y, int input_rms, float eps, void *workspace,
+                         int64_t workspace_bytes, hipStream_t s);
 // decode-step kernels around the linears (decode_step.hip)
 int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s);
 int bs_launch_attention_decode(const half_t *qkv, half_t *kcache, half_t *vcache, const half_t *cos, const half_t *sin,

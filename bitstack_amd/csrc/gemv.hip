@@ -434,6 +434,12 @@ struct RedMat {
 struct RedGroup {
     RedMat m[GEMV_MAX_GROUP];
     int n, mode;
+    // input RMS scale: when xin is set, every sum is multiplied by rsqrt(mean(xin[t, :]^2) + eps)
+    // before the bias - the scalar half of an RMSNorm in front of the matrices (its weight
+    // vector belongs folded into vt by the caller)
+    const half_t *xin;
+    int n_in;
+    float eps;
 };
 
 // Sum of the partials of output m of one matrix that this thread's slice covers.
@@ -503,18 +509,40 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
         if (r.bias) extra = (float)r.bias[m];
         if (grp.mode == EPI_RESIDUAL) res = (float)residual[(int64_t)t * ldy + r.y_off + m];
     }
+    float scale = 1.f;
+    __shared__ float ssq[RED_OUT * RED_SL / 64];
+    if (grp.xin) {                               // sum of squares of this token's input row, every workgroup for itself
+        const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
+        float q = 0.f;
+        for (int c = threadIdx.x * 8; c < grp.n_in; c += RED_OUT * RED_SL * 8) {
+            const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
+#pragma unroll
+            for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o, 64);
+        if ((threadIdx.x & 63) == 0) ssq[threadIdx.x >> 6] = q;
+    }
     __syncthreads();
+    if (grp.xin) {
+        float q = 0.f;
+#pragma unroll
+        for (int w = 0; w < RED_OUT * RED_SL / 64; w++) q += ssq[w];
+        scale = rsqrtf(q / (float)grp.n_in + grp.eps);
+    }
     red[0][ks][lo] = live ? slice_sum_any(r, T, t, m, ks, nks[0]) : 0.f;
     if (two) red[1][ks][lo] = live ? slice_sum_any(grp.m[1], T, t, m, ks, nks[1]) : 0.f;
     __syncthreads();
     if (ks != 0 || !live) return;
-    float s0 = extra;
+    float s0 = 0.f;
 #pragma unroll
     for (int k = 0; k < RED_SL; k++) s0 += red[0][k][lo];
+    s0 = s0 * scale + extra;
     if (two) {
-        float s1 = grp.m[1].bias ? (float)grp.m[1].bias[m] : 0.f;
+        float s1 = 0.f;
 #pragma unroll
         for (int k = 0; k < RED_SL; k++) s1 += red[1][k][lo];
+        s1 = s1 * scale + (grp.m[1].bias ? (float)grp.m[1].bias[m] : 0.f);
         const float gate = (float)(half_t)s0, up = (float)(half_t)s1;
         const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
         y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
@@ -639,7 +667,7 @@ bool gemv_shape_ok(int I, int M, int N, int T) {
 int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
 
 int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int mode, const half_t *residual,
-                 half_t *y, void *workspace, int64_t workspace_bytes, hipStream_t s) {
+                 half_t *y, bool input_rms, float eps, void *workspace, int64_t workspace_bytes, hipStream_t s) {
     if (a.n < 1 || a.n > GEMV_MAX_GROUP) return BS_ERR_SHAPE;
     if (!bs_aligned(x, 16)) return BS_ERR_SHAPE;
     int ldy = 0;
@@ -660,6 +688,9 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
     RedGroup r;
     g.n = r.n = a.n;
     r.mode = mode;
+    r.xin = nullptr;
+    r.n_in = N;
+    r.eps = eps;
     int y_off = 0, blocks = 0;
     for (int j = 0; j < a.n; j++) {
         g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
@@ -682,6 +713,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         if (st != BS_OK) return st;
         // the partial areas are laid out for tp tokens; a shorter last pass uses its own stride
         RedGroup rr = r;
+        if (input_rms) rr.xin = xp;
         int nblocks = blocks;
         if (tn != tp) {
             nblocks = 0;
@@ -736,13 +768,13 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
     GroupArgs a;
     a.n = 1;
     a.packed[0] = packed; a.u[0] = u; a.vt[0] = vt; a.bias[0] = bias; a.I[0] = I; a.M[0] = M;
-    return launch_group(a, N, K, x, T, EPI_NONE, nullptr, y, workspace, workspace_bytes, s);
+    return launch_group(a, N, K, x, T, EPI_NONE, nullptr, y, false, 0.f, workspace, workspace_bytes, s);
 }
 
 int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
                          const half_t *const *bias, const int *I, const int *M, int N, int K, const half_t *x, int T,
-                         int mode, const half_t *residual, half_t *y, void *workspace, int64_t workspace_bytes,
-                         hipStream_t s) {
+                         int mode, const half_t *residual, half_t *y, int input_rms, float eps, void *workspace,
+                         int64_t workspace_bytes, hipStream_t s) {
     if (n < 1 || n > GEMV_MAX_GROUP) return BS_ERR_SHAPE;
     if (mode == EPI_RESIDUAL && !residual) return BS_ERR_NULL;
     GroupArgs a;
@@ -751,5 +783,5 @@ int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *cons
         a.packed[j] = packed[j]; a.u[j] = u[j]; a.vt[j] = vt[j]; a.bias[j] = bias ? bias[j] : nullptr;
         a.I[j] = I[j]; a.M[j] = M[j];
     }
-    return launch_group(a, N, K, x, T, mode, residual, y, workspace, workspace_bytes, s);
+    return launch_group(a, N, K, x, T, mode, residual, y, input_rms != 0, eps, workspace, workspace_bytes, s);
 }

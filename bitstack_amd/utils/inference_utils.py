@@ -127,11 +127,13 @@ class MatrixGroup:
         return self._need[T]
 
 
-def bitstack_forward_group_hip(group: MatrixGroup, x, epilogue=_lib.EPI_NONE, residual=None, out=None):
+def bitstack_forward_group_hip(group: MatrixGroup, x, epilogue=_lib.EPI_NONE, residual=None, out=None, rms_eps=None):
     """All matrices of `group` applied to x [T, N] (T <= 8) in one launch pair, with
     the outputs side by side [T, sum M] (EPI_NONE), plus `residual` (EPI_RESIDUAL),
     or silu(first) * second [T, M] (EPI_SWIGLU).  What three (two) module calls and
-    the element-wise ops after them do in a decoder layer."""
+    the element-wise ops after them do in a decoder layer.  With rms_eps set, x is
+    the un-normalised row and every output is scaled by rsqrt(mean(x^2) + rms_eps)
+    (the norm's weight vector must already be folded into the group's vt)."""
     dev = _lib.require_gpu(x, residual, out)
     x2 = _f16c(x).view(-1, group.N)
     T = x2.shape[0]
@@ -148,9 +150,14 @@ def bitstack_forward_group_hip(group: MatrixGroup, x, epilogue=_lib.EPI_NONE, re
         raise ValueError("out must be a contiguous fp16 [T, width] tensor")
     ws = _lib.workspace(dev, need)
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().bs_forward_group(group.arr, group.n, group.N, group.K, _lib.ptr(x2), T, epilogue,
-                                               _lib.ptr(residual), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
-                                               _lib.stream_ptr(dev)), "bs_forward_group")
+        if rms_eps is None:
+            _lib.check(_lib.lib().bs_forward_group(group.arr, group.n, group.N, group.K, _lib.ptr(x2), T, epilogue,
+                                                   _lib.ptr(residual), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                                                   _lib.stream_ptr(dev)), "bs_forward_group")
+        else:
+            _lib.check(_lib.lib().bs_forward_group_rms(group.arr, group.n, group.N, group.K, _lib.ptr(x2), T, float(rms_eps),
+                                                       epilogue, _lib.ptr(residual), _lib.ptr(y), _lib.ptr(ws), ws.numel(),
+                                                       _lib.stream_ptr(dev)), "bs_forward_group_rms")
     return y
 
 

@@ -108,8 +108,8 @@ class SyntheticLlamaDecoder:
                   call per projection (the structure the reference runs);
     step_fused()  four launch pairs per layer for the seven linears (q/k/v in one,
                   o with the residual add, gate/up with the SiLU product, down with
-                  the residual add), one RMSNorm and one attention kernel between
-                  them, all from the library."""
+                  the residual add; the two RMSNorms ride on the q/k/v and gate/up
+                  launches) and one attention kernel, all from the library."""
 
     def __init__(self, shape: LlamaShape, config: dict, max_len: int, device, seed=0, batch=1):
         dev = torch.device(device)
@@ -249,14 +249,26 @@ class SyntheticLlamaDecoder:
         self.pos.add_(1)
 
     def _build_groups(self):
+        """Argument blocks of the grouped launches.  The RMSNorm weight vectors in front of
+        q/k/v and gate/up are folded into copies of those matrices' vt once
+        (vt_i[r, n] * weight[n]); the scalar rsqrt(mean(x^2) + eps) is applied by the
+        launch itself, so the fused step has no RMSNorm kernel inside a layer."""
         s, B = self.s, self.batch
         self._groups = []
+
+        def folded(mods, weight):
+            mats = []
+            for m in mods:
+                q, u, vt = m._stacked()
+                mats.append((q, u, (vt.float() * weight.float().view(1, 1, -1)).half(), m.bias))
+            return MatrixGroup(mats)
+
         for L in range(s.layers):
             lin = self.lin[L]
             self._groups.append({
-                "qkv": MatrixGroup.from_modules([lin["self_attn.q_proj"], lin["self_attn.k_proj"], lin["self_attn.v_proj"]]),
+                "qkv": folded([lin["self_attn.q_proj"], lin["self_attn.k_proj"], lin["self_attn.v_proj"]], self.norm_w[L, 0]),
                 "o": MatrixGroup.from_modules([lin["self_attn.o_proj"]]),
-                "gate_up": MatrixGroup.from_modules([lin["mlp.gate_proj"], lin["mlp.up_proj"]]),
+                "gate_up": folded([lin["mlp.gate_proj"], lin["mlp.up_proj"]], self.norm_w[L, 1]),
                 "down": MatrixGroup.from_modules([lin["mlp.down_proj"]]),
             })
         f16 = dict(dtype=torch.float16, device=self.dev)
@@ -277,13 +289,11 @@ class SyntheticLlamaDecoder:
         torch.index_select(self.embed, 0, self.token, out=xa)
         for L in range(s.layers):
             grp = self._groups[L]
-            rmsnorm_hip(xa, self.norm_w[L, 0], s.rms_eps, out=self._hn)
-            bitstack_forward_group_hip(grp["qkv"], self._hn, EPI_NONE, out=self._qkv)
+            bitstack_forward_group_hip(grp["qkv"], xa, EPI_NONE, out=self._qkv, rms_eps=s.rms_eps)
             attention_decode_hip(self._qkv, self.kcache[L], self.vcache[L], self.cos, self.sin, self.pos,
                                  s.heads, s.kv_heads, out=self._ctx)
             bitstack_forward_group_hip(grp["o"], self._ctx, EPI_RESIDUAL, residual=xa, out=xb)
-            rmsnorm_hip(xb, self.norm_w[L, 1], s.rms_eps, out=self._hn)
-            bitstack_forward_group_hip(grp["gate_up"], self._hn, EPI_SWIGLU, out=self._act)
+            bitstack_forward_group_hip(grp["gate_up"], xb, EPI_SWIGLU, out=self._act, rms_eps=s.rms_eps)
             bitstack_forward_group_hip(grp["down"], self._act, EPI_RESIDUAL, residual=xb, out=xa)
         rmsnorm_hip(xa, self.final_norm, s.rms_eps, out=self._hn)
         self.logits = F.linear(self._hn, self.lm_head)

@@ -164,6 +164,19 @@ int bs_forward_group(const bs_matrix *mats, int n, int N, int K, const void *x, 
                      void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * The same with an RMSNorm in front, without a launch for it: x is the
+ * UN-normalised row, every output is multiplied by rsqrt(mean(x[t, :]^2) + eps)
+ * before the bias (each workgroup of the reduce kernel recomputes that scalar),
+ * and the norm's weight vector is expected folded into the matrices by the
+ * caller (vt_i[r, n] * weight[n], done once).  input_layernorm -> q/k/v and
+ * post_attention_layernorm -> gate/up of a decoder layer then cost no kernel
+ * of their own.
+ */
+int bs_forward_group_rms(const bs_matrix *mats, int n, int N, int K, const void *x, int T, float eps,
+                         int epilogue, const void *residual, void *y,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * y[T, H] = weight o fp16( x * rsqrt(mean(x^2) + eps) ), statistics in fp32:
  * the RMSNorm in front of the attention and MLP linears of a decoder layer
  * (the reference leaves it to the Hugging Face model it patches,

@@ -256,3 +256,34 @@ def test_decoder_round_trips_through_a_checkpoint(tmp_path):
         assert torch.equal(a.logits, b.logits)
         assert not torch.equal(a.logits, small.logits)
     assert torch.equal(a.token, b.token)
+
+
+@pytest.mark.parametrize("shapes,N,T,mode", [([(3, 512), (2, 128), (2, 128)], 1024, 1, "none"),
+                                              ([(2, 4096), (3, 1024), (1, 1024)], 4096, 1, "none"),
+                                              ([(2, 1024), (3, 1024)], 2048, 1, "swiglu"),
+                                              ([(2, 256), (1, 256)], 512, 5, "swiglu"),
+                                              ([(2, 300)], 1536, 3, "none")])
+def test_group_forward_with_input_rms(shapes, N, T, mode):
+    """bs_forward_group_rms: the RMSNorm in front of the matrices without a launch of its own.  The
+    caller folds the norm weight into vt; the launch scales by rsqrt(mean(x^2) + eps)."""
+    print(f"group rms {shapes} N={N} T={T} {mode}", flush=True)
+    g = torch.Generator().manual_seed(N + T)
+    wn = (1 + 0.3 * torch.randn(N, generator=g)).half()
+    x = (torch.randn(T, N, generator=g) * 4).half()                       # far from unit RMS on purpose
+    eps = 1e-5
+    hn = LO.rmsnorm(x.double().numpy(), wn.double().numpy(), eps)         # float64 normalised input
+    mats, refs = [], []
+    for j, (I, M) in enumerate(shapes):
+        q, u, vt, _ = synthetic_layer(M, N, I, T, seed=40 + j, signed_factors=True)
+        b = (torch.randn(M, generator=g) * 0.05).half() if j % 2 == 0 else None
+        w = O.reconstruct_w_exact(q.numpy(), u.numpy(), vt.numpy())
+        refs.append(hn @ w.T + (0 if b is None else b.double().numpy()))
+        vt_folded = (vt.float() * wn.float().view(1, 1, -1)).half()
+        mats.append((q.to(dev()), u.to(dev()), vt_folded.to(dev()), None if b is None else b.to(dev())))
+    grp = IU.MatrixGroup(mats)
+    if mode == "swiglu":
+        y = IU.bitstack_forward_group_hip(grp, x.to(dev()), _lib.EPI_SWIGLU, rms_eps=eps).cpu().numpy()
+        assert_close(y, LO.silu(refs[0]) * refs[1], "rms + swiglu vs fp64", 2e-2, 3e-3)
+    else:
+        y = IU.bitstack_forward_group_hip(grp, x.to(dev()), rms_eps=eps).cpu().numpy()
+        assert_close(y, np.concatenate(refs, axis=1), "rms group vs fp64", 1e-2, 2e-3)
