@@ -53,12 +53,12 @@ __global__ __launch_bounds__(RMS_THREADS) void rmsnorm_kernel(const half_t *__re
     }
 }
 
-// One workgroup per (query head, sequence).  256 threads = 16 groups of 16 lanes;
-// a group walks every 16th cached position, a lane owns 8 of the 128 dimensions
+// One workgroup per (query head, sequence).  1024 threads = 64 groups of 16 lanes;
+// a group walks every 64th cached position, a lane owns 8 of the 128 dimensions
 // (one 16-byte load per cached row and lane, a row is one contiguous 256 bytes).
 // One pass: k and v of four positions are fetched together and folded into a
-// running (max, sum, weighted v) per group; the 16 groups are merged through LDS.
-constexpr int ATT_THREADS = 256, ATT_D = 128, ATT_MAX_LEN = 8192;
+// running (max, sum, weighted v) per group; the 64 groups are merged through LDS.
+constexpr int ATT_THREADS = 1024, ATT_GROUPS = ATT_THREADS / 16, ATT_D = 128, ATT_MAX_LEN = 8192;
 
 __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     const half_t *__restrict__ qkv, half_t *__restrict__ kcache, half_t *__restrict__ vcache,
@@ -66,8 +66,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     half_t *__restrict__ out, int heads, int kv_heads, int max_len) {
     __shared__ float qs[ATT_D];                  // rotated query, pre-scaled
     __shared__ __attribute__((aligned(16))) half_t knew[ATT_D], vnew[ATT_D];   // this position's rotated k and v
-    __shared__ float gm[16], gl[16];             // per group: running max, sum of exp
-    __shared__ float accs[16][ATT_D];
+    __shared__ float gm[ATT_GROUPS], gl[ATT_GROUPS];             // per group: running max, sum of exp
+    __shared__ float accs[ATT_GROUPS][ATT_D];
     const int tid = threadIdx.x, lane16 = tid & 15, grp = tid >> 4;
     const int head = blockIdx.x, b = blockIdx.y;
     const int rep = heads / kv_heads, hk = head / rep;
@@ -131,18 +131,18 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
         for (int e = 0; e < 8; e++) acc[e] = acc[e] * r + w * (float)v8[e];
         m = mn;
     };
-    for (int p0 = grp; p0 < pos; p0 += 64) {
+    for (int p0 = grp; p0 < pos; p0 += 4 * ATT_GROUPS) {
         half8_t k8[4], v8[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int p = min(p0 + 16 * j, pos - 1);
+            const int p = min(p0 + ATT_GROUPS * j, pos - 1);
             k8[j] = *reinterpret_cast<const half8_t *>(kc + (int64_t)p * ATT_D + 8 * lane16);
             v8[j] = *reinterpret_cast<const half8_t *>(vc + (int64_t)p * ATT_D + 8 * lane16);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const float sc = score_of(k8[j]);
-            if (p0 + 16 * j < pos) fold(sc, v8[j]);
+            if (p0 + ATT_GROUPS * j < pos) fold(sc, v8[j]);
         }
     }
     if (grp == 0)      // this step's own k and v, from LDS
@@ -155,10 +155,10 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     if (tid < ATT_D) {
         float mx = gm[0];
 #pragma unroll
-        for (int gq = 1; gq < 16; gq++) mx = fmaxf(mx, gm[gq]);
+        for (int gq = 1; gq < ATT_GROUPS; gq++) mx = fmaxf(mx, gm[gq]);
         float o = 0.f, den = 0.f;
 #pragma unroll
-        for (int gq = 0; gq < 16; gq++) {
+        for (int gq = 0; gq < ATT_GROUPS; gq++) {
             const float r = gl[gq] > 0.f ? __expf(gm[gq] - mx) : 0.f;     // groups that saw no position
             o += r * accs[gq][tid];
             den += r * gl[gq];
