@@ -42,6 +42,7 @@ SIGNATURES.update({
     "bs_forward_group_workspace_bytes": (_L, [_P, _I, _I, _I, _I]),
     "bs_forward_group": (_I, [_P, _I, _I, _I, _P, _I, _I, _P, _P, _P, _L, _P]),
     "bs_forward_group_rms": (_I, [_P, _I, _I, _I, _P, _I, ctypes.c_float, _I, _P, _P, _P, _L, _P]),
+    "bs_argmax_f16": (_I, [_P, _P, _I, _I, _P]),
     "bs_rmsnorm_f16": (_I, [_P, _P, _P, _I, _I, ctypes.c_float, _P]),
     "bs_attention_decode_f16": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
 })

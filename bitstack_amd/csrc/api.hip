@@ -161,3 +161,11 @@ extern "C" int bs_attention_decode_f16(const void *qkv, void *kcache, void *vcac
                                       (const half_t *)sin, pos, (half_t *)out, B, heads, kv_heads, head_dim, max_len,
                                       (hipStream_t)stream);
 }
+
+extern "C" int bs_argmax_f16(const void *x, int64_t *out, int B, int V, void *stream) {
+    if (B < 0 || V <= 0) return BS_ERR_SHAPE;
+    if (B == 0) return BS_OK;
+    if (!x || !out) return BS_ERR_NULL;
+    if (!bs_aligned(x, 16) || !bs_aligned(out, 8) || (B > 1 && V % 8 != 0)) return BS_ERR_ALIGN;
+    return bs_launch_argmax((const half_t *)x, out, B, V, (hipStream_t)stream);
+}

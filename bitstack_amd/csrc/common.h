@@ -51,6 +51,7 @@ int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *cons
                          int mode, const half_t *residual, half_t *y, int input_rms, float eps, void *workspace,
                          int64_t workspace_bytes, hipStream_t s);
 // decode-step kernels around the linears (decode_step.hip)
+int bs_launch_argmax(const half_t *x, int64_t *out, int B, int V, hipStream_t s);
 int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s);
 int bs_launch_attention_decode(const half_t *qkv, half_t *kcache, half_t *vcache, const half_t *cos, const half_t *sin,
                                const int64_t *pos, half_t *out, int B, int heads, int kv_heads, int head_dim,

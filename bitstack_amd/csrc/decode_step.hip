@@ -167,7 +167,52 @@ __global__ __launch_bounds__(ATT_THREADS) void attention_decode_kernel(
     }
 }
 
+// Greedy token: index of the largest of V fp16 values per row (the lowest index among
+// equals; NaN never wins), one workgroup per row.
+constexpr int ARG_THREADS = 1024;
+
+__global__ __launch_bounds__(ARG_THREADS) void argmax_kernel(const half_t *__restrict__ x, int64_t *__restrict__ out, int V) {
+    __shared__ float bv[ARG_THREADS / 64];
+    __shared__ int bi[ARG_THREADS / 64];
+    const int tid = threadIdx.x;
+    const half_t *row = x + (int64_t)blockIdx.x * V;
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    const int v8 = V & ~7;
+    for (int c = tid * 8; c < v8; c += ARG_THREADS * 8) {       // ascending per thread: a later equal value never replaces
+        const half8_t v = *reinterpret_cast<const half8_t *>(row + c);
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float f = (float)v[e];
+            if (f > best || (f == best && c + e < at)) { best = f; at = c + e; }
+        }
+    }
+    for (int c = v8 + tid; c < V; c += ARG_THREADS) {
+        const float f = (float)row[c];
+        if (f > best || (f == best && c < at)) { best = f; at = c; }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oa = __shfl_xor(at, o, 64);
+        if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if ((tid & 63) == 0) { bv[tid >> 6] = best; bi[tid >> 6] = at; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < ARG_THREADS / 64; w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < at)) { best = bv[w]; at = bi[w]; }
+        out[blockIdx.x] = at == 0x7fffffff ? 0 : at;            // a row of NaNs / -inf: index 0
+    }
+}
+
 }  // namespace
+
+int bs_launch_argmax(const half_t *x, int64_t *out, int B, int V, hipStream_t s) {
+    argmax_kernel<<<B, ARG_THREADS, 0, s>>>(x, out, V);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
 
 int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s) {
     if (H > RMS_THREADS * RMS_MAX_CHUNKS * 8) return BS_ERR_SHAPE;

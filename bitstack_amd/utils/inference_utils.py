@@ -198,6 +198,20 @@ def attention_decode_hip(qkv, kcache, vcache, cos, sin, pos, heads, kv_heads, ou
     return y
 
 
+def argmax_hip(x, out=None):
+    """Index of the largest value of every row of x [B, V] (fp16), int64 [B]."""
+    dev = _lib.require_gpu(x, out)
+    if x.dim() != 2 or x.dtype != torch.float16 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous fp16 [B, V] tensor")
+    y = out if out is not None else torch.empty(x.shape[0], dtype=torch.int64, device=dev)
+    if y.dtype != torch.int64 or y.numel() != x.shape[0] or not y.is_contiguous():
+        raise ValueError("out must be a contiguous int64 [B] tensor")
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().bs_argmax_f16(_lib.ptr(x), _lib.ptr(y), x.shape[0], x.shape[1], _lib.stream_ptr(dev)),
+                   "bs_argmax_f16")
+    return y
+
+
 def linear_f16_hip(x, w, bias=None):
     """F.linear on the library's own MFMA kernel (fp16 in, fp32 accumulate)."""
     dev = _lib.require_gpu(x, w, bias)

@@ -22,8 +22,8 @@ import torch.nn.functional as F
 
 from bitstack_amd._lib import EPI_NONE, EPI_RESIDUAL, EPI_SWIGLU
 from bitstack_amd.modules.BitStackLinear import BitStackLinear
-from bitstack_amd.utils.inference_utils import (MatrixGroup, attention_decode_hip, bitstack_forward_group_hip,
-                                                rmsnorm_hip)
+from bitstack_amd.utils.inference_utils import (MatrixGroup, argmax_hip, attention_decode_hip,
+                                                bitstack_forward_group_hip, rmsnorm_hip)
 
 PROJ = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
         "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")
@@ -297,7 +297,7 @@ class SyntheticLlamaDecoder:
             bitstack_forward_group_hip(grp["down"], self._act, EPI_RESIDUAL, residual=xb, out=xa)
         rmsnorm_hip(xa, self.final_norm, s.rms_eps, out=self._hn)
         self.logits = F.linear(self._hn, self.lm_head)
-        self.token.copy_(self.logits.argmax(-1))
+        argmax_hip(self.logits, out=self.token)
         self.pos.add_(1)
 
     def prefill_positions(self, prompt: torch.Tensor, fused=False):

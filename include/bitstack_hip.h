@@ -200,6 +200,14 @@ int bs_attention_decode_f16(const void *qkv, void *kcache, void *vcache, const v
                             const int64_t *pos, void *out, int B, int heads, int kv_heads, int head_dim,
                             int max_len, void *stream);
 
+/*
+ * out[b] = index of the largest of x[b, 0..V) (fp16; the lowest index among
+ * equal values): the greedy token of a decode step from the logits.  Rows must
+ * start 16-byte aligned (V % 8 == 0 when B > 1).  No counterpart in the
+ * reference (generation is left to Hugging Face code).
+ */
+int bs_argmax_f16(const void *x, int64_t *out, int B, int V, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

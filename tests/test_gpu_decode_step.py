@@ -287,3 +287,17 @@ def test_group_forward_with_input_rms(shapes, N, T, mode):
     else:
         y = IU.bitstack_forward_group_hip(grp, x.to(dev()), rms_eps=eps).cpu().numpy()
         assert_close(y, np.concatenate(refs, axis=1), "rms group vs fp64", 1e-2, 2e-3)
+
+
+@pytest.mark.parametrize("B,V", [(1, 128256), (3, 256), (2, 4096), (1, 13), (1, 8)])
+def test_argmax(B, V):
+    g = torch.Generator().manual_seed(V)
+    x = torch.randn(B, V, generator=g).half()
+    x[0, V // 2] = x[0].max()                       # a tie: the lower index must win
+    got = IU.argmax_hip(x.to(dev())).cpu()
+    want = torch.tensor([int(np.argmax(r)) for r in x.float().numpy()])     # numpy: first maximum
+    assert torch.equal(got, want)
+    x[0, 3] = float("nan")
+    got = IU.argmax_hip(x.to(dev())).cpu()
+    row = x[0].float().numpy().copy(); row[3] = -np.inf
+    assert int(got[0]) == int(np.argmax(row))       # NaN never wins

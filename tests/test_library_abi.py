@@ -109,6 +109,9 @@ def test_group_and_decode_step_validation(L):
     assert L.bs_forward_group(mats, 2, 512, 16, one, 1, 2, nul, one, one, big, nul) == -2       # SwiGLU needs equal M
     assert L.bs_forward_group_rms(mats, 2, 512, 16, nul, 1, 1e-5, 0, nul, one, one, big, nul) == -1
     assert L.bs_forward_group_rms(mats, 2, 512, 16, one, 1, -1.0, 0, nul, one, one, big, nul) == -2   # eps < 0
+    assert L.bs_argmax_f16(nul, one, 1, 64, nul) == -1
+    assert L.bs_argmax_f16(one, one, 1, 0, nul) == -2
+    assert L.bs_argmax_f16(one, one, 2, 13, nul) == -4
     # rmsnorm / attention
     assert L.bs_rmsnorm_f16(one, one, one, 1, 100, 1e-5, nul) == -2
     assert L.bs_rmsnorm_f16(one, one, one, 1, 32768, 1e-5, nul) == -2
