@@ -24,6 +24,21 @@ static inline bool bs_aligned(const void *p, uintptr_t a) {
 
 static inline int64_t bs_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Kernels that need more than 64 KB of dynamic LDS must be allowed to, once per kernel AND
+// per device (the attribute lives with the device's copy of the code).  `granted[d]` is the
+// size already allowed on device d; the caller keeps one such array per kernel.
+constexpr int BS_MAX_DEVICES = 64;
+static inline int bs_allow_lds(const void *kernel, size_t bytes, size_t *granted) {
+    if (bytes <= 64 * 1024) return BS_OK;
+    int dev = 0;
+    BS_HIP_TRY(hipGetDevice(&dev));
+    const bool tracked = dev >= 0 && dev < BS_MAX_DEVICES;
+    if (tracked && granted[dev] >= bytes) return BS_OK;
+    BS_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    if (tracked) granted[dev] = bytes;
+    return BS_OK;
+}
+
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));

@@ -242,14 +242,10 @@ int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y
                  hipStream_t s) {
     constexpr int BT = WT * AT * 32, BF = WF * AF * 32;
     constexpr size_t lds = (size_t)2 * (BT + BF) * (GK + 8) * sizeof(half_t);
-    static bool raised = false;
-    if (lds > 64 * 1024 && !raised) {
-        BS_HIP_TRY(hipFuncSetAttribute((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        BS_HIP_TRY(hipFuncSetAttribute((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        raised = true;
-    }
+    static size_t granted[2][BS_MAX_DEVICES] = {};
+    int st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>, lds, granted[0]);
+    if (st == BS_OK) st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>, lds, granted[1]);
+    if (st != BS_OK) return st;
     dim3 grid((unsigned)bs_cdiv(M, BF), (unsigned)bs_cdiv(T, BT));
     if (N % GK == 0)
         linear_f16_kernel<WT, WF, AT, AF, GK, false><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);

@@ -633,12 +633,9 @@ struct GroupArgs {          // host-side view of one call
 template <int T, int WAVES, int R>
 int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     const size_t lds = (size_t)2 * T * 16384 + (size_t)2 * WAVES * T * 64;
-    static bool raised = false;      // per instantiation; raising the limit is idempotent
-    if (lds > 64 * 1024 && !raised) {
-        BS_HIP_TRY(hipFuncSetAttribute((const void *)gemv_kernel<T, WAVES, R>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        raised = true;
-    }
+    static size_t granted[BS_MAX_DEVICES] = {};      // per instantiation
+    const int st = bs_allow_lds((const void *)gemv_kernel<T, WAVES, R>, lds, granted);
+    if (st != BS_OK) return st;
     gemv_kernel<T, WAVES, R><<<p.grid, 64 * WAVES, lds, s>>>(grp, x, N, K, p.n_chunks);
     BS_LAUNCH_CHECK();
     return BS_OK;
