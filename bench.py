@@ -50,8 +50,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
-    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill"], default=None,
+    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
+    ap.add_argument("--layer", default="14336x4096x16x1",
+                    help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
     return ap.parse_args()
 
@@ -273,6 +275,27 @@ def main():
             del lp
         return pre
 
+    if a.only == "one_layer":
+        # 12 forwards of ONE layer on 3 rotating copies of its buffers (as every layer of the sweep
+        # is run), nothing else on the GPU: the process to put under rocprofv3 --pmc
+        M, N, I, T = (int(v) for v in a.layer.split("x"))
+        copies = [Layer(M, N, I, T, seed, dev) for seed in range(3)]
+        ws = workspace_for(copies)
+        fns = [make_forward(L, lib, ws, stream) for L in copies]
+        for r in range(2):
+            fns[r % 3]()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for r in range(12):
+            fns[r % 3]()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / 12 * 1e3
+        print(json.dumps({"one_layer": {"M": M, "N": N, "I": I, "T": T, "algorithmic_bytes": copies[0].bytes,
+                                        "us_per_forward": round(us, 2), "GBps": round(copies[0].bytes / us / 1e3, 1),
+                                        "decode_plan": _lib.decode_plan(I, M, N, 16, T)}}))
+        return
     if a.only == "decode_8b":
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
         return
@@ -314,8 +337,8 @@ def main():
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     # HBM bytes per forward measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the largest launch of
     # that kernel (14336x4096, I=16), scaled by what the same counters read for a 256 MiB copy
-    # (FETCH_SIZE x2.0, WRITE_SIZE x1.0; profiles/gemv_traffic_counters.txt): 196 MB vs 126.9 MB algorithmic
-    traffic_ratio = 1.55
+    # (FETCH_SIZE x2.0, WRITE_SIZE x1.0; profiles/gemv_traffic_counters.txt): 205 MB vs 126.9 MB algorithmic
+    traffic_ratio = 1.62
 
     out = {
         "metric": "packed-sign GEMV HBM GB/s (decode sweep, Llama-3.1-8B linear shapes, T=1)",
@@ -334,7 +357,7 @@ def main():
                      "launches_per_step": dom_n,
                      "avg_us_per_launch": round(dom_ms * 1e3 / dom_n, 2),
                      "avg_algorithmic_bytes_per_launch": round(dom_bytes / dom_n),
-                     "traffic_note": "HBM bytes per launch = algorithmic x 1.55, the FETCH_SIZE+WRITE_SIZE ratio "
+                     "traffic_note": "HBM bytes per launch = algorithmic x 1.62, the FETCH_SIZE+WRITE_SIZE ratio "
                                      "measured on this kernel's largest launch (profiles/gemv_traffic_counters.txt)",
                      "whole_sweep_GBps_by_events": round(sweep_gbs, 1),
                      "best_layer": best},
