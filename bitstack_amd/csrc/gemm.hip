@@ -18,9 +18,19 @@
 // the few token rows); up to 32 tokens: linear_skinny_kernel (below).
 #include "common.h"
 #include <type_traits>
+#include <utility>
 
 namespace {
 
+// Compile-time loop (the index is a constant expression inside the body).
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 template <int WT, int WF, int AT, int AF, int GK, bool KTAIL>
 __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
@@ -76,65 +86,113 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     // the compiler's count of outstanding loads is exact and a wait for one set never
     // drains the other.  KTAIL (N not a multiple of GK): pieces beyond column N are read
     // from column 0 instead and replaced by zeros.
-    uint4_t stage[2][PER_THREAD];
-    auto fetch = [&](auto setc, int step_) {
-        constexpr int set = decltype(setc)::value;
+    uint4_t stage[3][PER_THREAD];
+    // part `part` of `parts` of the pieces of one step (the whole step: 0 of 1)
+    auto fetch = [&](auto setc, int step_, auto partc, auto partsc) {
+        constexpr int set = decltype(setc)::value, part = decltype(partc)::value, parts = decltype(partsc)::value;
+        constexpr int j0 = part * PER_THREAD / parts, j1 = (part + 1) * PER_THREAD / parts;
         const int step = min(step_, steps - 1);
         if constexpr (KTAIL) {
             const bool in = step * GK + 8 * lpiece < N;              // N % 8 == 0: a piece is all in or all out
             const uint32_t koff = in ? (uint32_t)step * (GK * 2) : 0u - 16u * lpiece;
 #pragma unroll
-            for (int j = 0; j < PER_THREAD; j++) {
+            for (int j = j0; j < j1; j++) {
                 const uint4_t v = *reinterpret_cast<const uint4_t *>((j < JX ? xt : wt_) + (off[j] + koff));
                 stage[set][j] = in ? v : (uint4_t){0, 0, 0, 0};
             }
         } else {
             const char *xs = xt + (int64_t)step * (GK * 2), *ws = wt_ + (int64_t)step * (GK * 2);
 #pragma unroll
-            for (int j = 0; j < PER_THREAD; j++)
+            for (int j = j0; j < j1; j++)
                 stage[set][j] = *reinterpret_cast<const uint4_t *>((j < JX ? xs : ws) + off[j]);
         }
     };
-    auto stash = [&](auto setc, int buf) {
-        constexpr int set = decltype(setc)::value;
+    // part `part` of `parts` of a register set goes to LDS (the whole set: 0 of 1)
+    auto stash = [&](auto setc, int buf, auto partc, auto partsc) {
+        constexpr int set = decltype(setc)::value, part = decltype(partc)::value, parts = decltype(partsc)::value;
 #pragma unroll
-        for (int j = 0; j < PER_THREAD; j++) *reinterpret_cast<uint4_t *>(&lds[buf][dst[j]]) = stage[set][j];
+        for (int j = part * PER_THREAD / parts; j < (part + 1) * PER_THREAD / parts; j++)
+            *reinterpret_cast<uint4_t *>(&lds[buf][dst[j]]) = stage[set][j];
     };
-    auto multiply = [&](int buf) {
+    // Fragments travel through two register sets as well: the LDS reads of sub-step
+    // kk + 1 are issued before the MFMAs of sub-step kk, and those of the next step's
+    // first sub-step right after the barrier, before the MFMAs of this step's last one
+    // (whose fragments were read before the barrier, so the buffer is free to be
+    // overwritten).  No MFMA waits for an LDS read issued just before it.
+    constexpr int NK = GK / 16;
+    static_assert(NK % 2 == 0, "the fragment sets alternate with a period of two sub-steps");
+    half8_t fa[2][AT], fb[2][AF];
+    auto load_frags = [&](auto setc, int buf, int kk) {
+        constexpr int set = decltype(setc)::value;
         const half_t *xs = &lds[buf][0], *ws = &lds[buf][BT * LSTRIDE];
 #pragma unroll
-        for (int kk = 0; kk < GK / 16; kk++) {
-            half8_t a[AT], b[AF];
+        for (int j = 0; j < AT; j++)
+            fa[set][j] = *reinterpret_cast<const half8_t *>(xs + (wt + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
 #pragma unroll
-            for (int j = 0; j < AT; j++)
-                a[j] = *reinterpret_cast<const half8_t *>(xs + (wt + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
+        for (int j = 0; j < AF; j++)
+            fb[set][j] = *reinterpret_cast<const half8_t *>(ws + (wf + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
+    };
+    auto mfmas = [&](auto setc) {
+        constexpr int set = decltype(setc)::value;
 #pragma unroll
-            for (int j = 0; j < AF; j++)
-                b[j] = *reinterpret_cast<const half8_t *>(ws + (wf + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
+        for (int ai = 0; ai < AT; ai++)
 #pragma unroll
-            for (int ai = 0; ai < AT; ai++)
-#pragma unroll
-                for (int bi = 0; bi < AF; bi++)
-                    acc[ai][bi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ai], b[bi], acc[ai][bi], 0, 0, 0);
-        }
+            for (int bi = 0; bi < AF; bi++)
+                acc[ai][bi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][ai], fb[set][bi], acc[ai][bi], 0, 0, 0);
     };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     // step s reads LDS buffer s & 1; its pieces travelled through register set s & 1
-    auto one_step = [&](auto cur, auto nxt, int step) {
-        fetch(cur, step + 2);                                 // set `cur` was emptied into LDS a step ago
-        multiply(step & 1);
-        stash(nxt, (step + 1) & 1);                           // after the last step: a copy nobody reads
+    // Neither the requests for step s + 2 nor the LDS writes of step s + 1 (requested a
+    // step ago) are issued in one burst - a wave that queues six or more 1 KB requests
+    // blocks on the address unit and every wave of the workgroup does so at the same
+    // time, right after the barrier, with the matrix pipe idle.  Both are cut into
+    // portions, one per group of MFMAs, issued together with the fragment reads in front
+    // of the group.  Nobody reads the other LDS buffer between the previous barrier and
+    // the next one, so it can be written all along the step.
+    using PF = std::integral_constant<int, NK>;
+    using PS = std::integral_constant<int, NK - 1>;
+    using S2 = std::integral_constant<int, 2>;
+    auto one_step = [&](auto cur, auto nxt, auto bufc, int step) {
+        constexpr int buf = decltype(bufc)::value;
+        static_for<NK / 2>([&](auto hc) {
+            constexpr int kk = 2 * decltype(hc)::value;
+            fetch(cur, step + 3, std::integral_constant<int, kk>{}, PF{});   // set `cur` was emptied into LDS a step ago
+            load_frags(S1{}, buf, kk + 1);
+            stash(nxt, buf ^ 1, std::integral_constant<int, kk>{}, PS{});    // after the last step: a copy nobody reads
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas(S0{});
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (kk + 2 < NK) {
+                fetch(cur, step + 3, std::integral_constant<int, kk + 1>{}, PF{});
+                load_frags(S0{}, buf, kk + 2);
+                stash(nxt, buf ^ 1, std::integral_constant<int, kk + 1>{}, PS{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfmas(S1{});
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
         __syncthreads();
+        fetch(cur, step + 3, std::integral_constant<int, NK - 1>{}, PF{});
+        load_frags(S0{}, buf ^ 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(S1{});
+        __builtin_amdgcn_sched_barrier(0);
     };
 
-    fetch(S0{}, 0);
-    fetch(S1{}, 1);
-    stash(S0{}, 0);
+    fetch(S0{}, 0, S0{}, S1{});
+    fetch(S1{}, 1, S0{}, S1{});
+    fetch(S2{}, 2, S0{}, S1{});
+    stash(S0{}, 0, S0{}, S1{});
     __syncthreads();
-    for (int step = 0; step < steps; step += 2) {
-        one_step(S0{}, S1{}, step);
-        if (step + 1 < steps) one_step(S1{}, S0{}, step + 1);
+    load_frags(S0{}, 0, 0);
+    for (int step = 0; step < steps; step += 6) {
+        one_step(S0{}, S1{}, S0{}, step);
+        if (step + 1 < steps) one_step(S1{}, S2{}, S1{}, step + 1);
+        if (step + 2 < steps) one_step(S2{}, S0{}, S0{}, step + 2);
+        if (step + 3 < steps) one_step(S0{}, S1{}, S1{}, step + 3);
+        if (step + 4 < steps) one_step(S1{}, S2{}, S0{}, step + 4);
+        if (step + 5 < steps) one_step(S2{}, S0{}, S1{}, step + 5);
     }
 
     // D[token, feature]: lane holds feature l32, tokens 8 * (v / 4) + 4 * kh + v % 4
@@ -267,7 +325,8 @@ int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, h
                            : launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
         } else {
             // 128 x 256 tiles (8 waves) once they still give every CU a workgroup, else 128 x 128
-            st = bs_cdiv(T, 128) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s)
+            st = bs_cdiv(T, 256) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s) :
+                 bs_cdiv(T, 128) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s)
                                                              : launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
         }
         if (st != BS_OK) return st;
