@@ -5,15 +5,26 @@
 // row (A = tokens) or one column (B = features), i.e. one 16-byte read per
 // fragment.
 //
-// More than 128 tokens: linear_f16_kernel, 2 x 2 (or 2 x 4) waves of 2 x 2 MFMA tiles
-// (128 tokens x 128 or 256 features per workgroup), k-steps of 64 columns through
-// LDS; rows are padded by 8 halves so that the eight lanes served per LDS cycle hit
-// disjoint banks.  Global loads run two k-steps ahead of the MFMAs through two
-// register sets, all of them unconditional with a scalar base and a 32-bit lane
-// offset (no address arithmetic or selects in the loop); two LDS buffers, one
-// barrier per step.  Measured dead ends: 32-column steps, 128 x 64 and 128 x 128
-// per-wave tiles (the compiler's register allocation collapses), 256 x 256
-// workgroup tiles with 16 waves.
+// More than 128 tokens: linear_f16_kernel, WT x WF waves of AT x AF MFMA tiles each,
+// k-steps of GK columns through two LDS buffers; rows are padded by 8 halves so that
+// the lanes served per LDS cycle hit disjoint banks.  Four shapes are instantiated:
+// 256 x 256 (8 waves of 128 x 64, GK = 32) and 128 x 256 (8 waves of 64 x 64) for
+// grids that cover the chip, 128 x 128 and 64 x 64 (4 waves, two workgroups per CU,
+// the latter with GK = 128: half as many barriers) for the smaller ones; the launcher
+// takes the largest tile whose grid still has about 160 workgroups.
+// The loop is software-pipelined at three levels, all through registers:
+//   - global requests run three k-steps ahead through three register sets, all of
+//     them unconditional with a scalar base and a 32-bit lane offset;
+//   - the LDS writes of step s + 1 and the requests of step s + 3 are cut into one
+//     portion per MFMA group instead of one burst per step;
+//   - MFMA fragments are read from LDS one group ahead of use, the first group of the
+//     next step right behind the barrier.
+// One barrier per step.  On this part LDS takes b128 reads at about 460 B/ns per CU
+// and b128 writes at about 165 B/ns (independent of the lane-to-address map as long as
+// rows are padded), global requests at 64 B per clock: with 64 x 64 per-wave tiles the
+// LDS time equals the MFMA time, which is what the larger tiles are for.  Measured dead
+// ends: 128 x 128 per-wave tiles with one wave per SIMD (nothing covers a wait), a
+// per-workgroup rotation of the k order (less sharing in L2), 16-wave workgroups.
 // 33..128 tokens use narrower workgroups of the same kernel (more workgroups for
 // the few token rows); up to 32 tokens: linear_skinny_kernel (below).
 #include "common.h"
@@ -324,10 +335,14 @@ int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, h
             st = M >= 8192 ? launch_tiled<2, 2, 2, 1, 64>(x, w, bias, y, T, M, N, s)
                            : launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
         } else {
-            // 128 x 256 tiles (8 waves) once they still give every CU a workgroup, else 128 x 128
-            st = bs_cdiv(T, 256) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s) :
-                 bs_cdiv(T, 128) * bs_cdiv(M, 256) >= 256 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s)
-                                                             : launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+            // The largest tile whose grid still covers most of the 256 CUs: 256 x 256 and
+            // 128 x 256 (8 waves) move the fewest bytes per flop; 128 x 128 and 64 x 64
+            // (4 waves, two workgroups per CU) keep a small problem spread over the chip.
+            const auto wgs = [&](int bt, int bf) { return bs_cdiv(T, bt) * bs_cdiv(M, bf); };
+            st = wgs(256, 256) >= 160 ? launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s) :
+                 wgs(128, 256) >= 160 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s) :
+                 wgs(128, 128) >= 192 ? launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s)
+                                      : launch_tiled<2, 2, 1, 1, 128>(x, w, bias, y, T, M, N, s);
         }
         if (st != BS_OK) return st;
     } else {
