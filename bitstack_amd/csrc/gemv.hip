@@ -663,10 +663,76 @@ bool gemv_shape_ok(int I, int M, int N, int T) {
 // Tokens are processed in passes of at most four (LDS holds Z for four tokens).
 int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
 
+// From this many tokens on the strip kernel (weight patches rebuilt in registers and
+// multiplied at once) is faster than passes of the factor-through kernel, which needs 16
+// rank-MFMAs per token and patch where the strip kernel needs one for 16 tokens.
+constexpr int STRIP_MIN_T = 5, STRIP_MAX_T = 32;
+
+bool strip_group_ok(const int *I, const int *M, int n, int N, int K, int T) {
+    for (int j = 0; j < n; j++)
+        if (bs_strip_partials(I[j], M[j], N, K, T) == 0) return false;
+    return true;
+}
+bool gemv_group_ok(const int *I, const int *M, int n, int N, int T) {
+    for (int j = 0; j < n; j++)
+        if (!gemv_shape_ok(I[j], M[j], N, T)) return false;
+    return true;
+}
+// 1: strip kernel, 0: factor-through kernel, -1: neither takes the shapes
+int group_path(const int *I, const int *M, int n, int N, int K, int T) {
+    if (n < 1 || n > GEMV_MAX_GROUP) return -1;
+    if (T >= STRIP_MIN_T && T <= STRIP_MAX_T && strip_group_ok(I, M, n, N, K, T)) return 1;
+    if (gemv_group_ok(I, M, n, N, T)) return 0;
+    return -1;
+}
+int64_t strip_part_floats(const int *I, const int *M, int n, int N, int K, int T) {
+    int64_t total = 0;
+    for (int j = 0; j < n; j++) total += (int64_t)bs_strip_partials(I[j], M[j], N, K, T) * T * M[j];
+    return total;
+}
+
+// Strip path: one launch per matrix writes part[strip, t, m]; the reduce kernel reads that
+// as "one partial per block" with the strips in the place of the blocks.
+int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T, int mode, const half_t *residual,
+                        half_t *y, bool input_rms, float eps, void *workspace, int64_t workspace_bytes, hipStream_t s) {
+    if (!workspace || workspace_bytes < strip_part_floats(a.I, a.M, a.n, N, K, T) * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
+    float *part = (float *)workspace;
+    RedGroup r;
+    r.n = a.n;
+    r.mode = mode;
+    r.xin = input_rms ? x : nullptr;
+    r.n_in = N;
+    r.eps = eps;
+    int ldy = 0, blocks = 0;
+    int64_t off = 0;
+    for (int j = 0; j < a.n; j++) {
+        const int st = bs_launch_strip_partials(a.packed[j], a.u[j], a.vt[j], x, part + off, a.I[j], a.M[j], N, K, T, s);
+        if (st != BS_OK) return st;
+        const int groups = bs_strip_partials(a.I[j], a.M[j], N, K, T);
+        r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], (int)bs_cdiv(a.M[j], RED_OUT), 1, ldy, blocks, Split{1, 0}};
+        off += (int64_t)groups * T * a.M[j];
+        ldy += a.M[j];
+        if (mode != EPI_SWIGLU || j == 0) blocks += T * (int)bs_cdiv(a.M[j], RED_OUT);
+    }
+    if (mode == EPI_SWIGLU) ldy = a.M[0];
+    for (int j = a.n; j < GEMV_MAX_GROUP; j++) r.m[j] = r.m[0];
+    gemv_reduce_kernel<<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, RED_OUT, 1);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
 int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int mode, const half_t *residual,
                  half_t *y, bool input_rms, float eps, void *workspace, int64_t workspace_bytes, hipStream_t s) {
     if (a.n < 1 || a.n > GEMV_MAX_GROUP) return BS_ERR_SHAPE;
     if (!bs_aligned(x, 16)) return BS_ERR_SHAPE;
+    if (mode == EPI_SWIGLU && (a.n != 2 || a.M[0] != a.M[1])) return BS_ERR_SHAPE;
+    const int path = group_path(a.I, a.M, a.n, N, K, T);
+    if (path < 0) return BS_ERR_SHAPE;
+    if (path == 1) {
+        for (int j = 0; j < a.n; j++)
+            if (!bs_aligned(a.packed[j], 16) || !bs_aligned(a.vt[j], 16) || !bs_aligned(a.u[j], 8)) return BS_ERR_SHAPE;
+        return launch_group_strips(a, N, K, x, T, mode, residual, y, input_rms, eps, workspace, workspace_bytes, s);
+    }
     int ldy = 0;
     for (int j = 0; j < a.n; j++) {
         if (!gemv_shape_ok(a.I[j], a.M[j], N, T)) return BS_ERR_SHAPE;
@@ -730,17 +796,15 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
 }  // namespace
 
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T) {
-    (void)K;
-    if (!gemv_shape_ok(I, M, N, T)) return 0;
-    const Plan p = make_plan(&I, &M, 1, N, pass_tokens(T));
-    return p.part_total * (int64_t)sizeof(float);
+    return bs_gemv_group_workspace_bytes(&I, &M, 1, N, K, T);
 }
 
+// Bytes of scratch the packed-sign paths (factor-through or strip kernel) need for these
+// matrices and token count; 0 when neither takes them.
 int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, int K, int T) {
-    (void)K;
-    if (n < 1 || n > GEMV_MAX_GROUP) return 0;
-    for (int j = 0; j < n; j++)
-        if (!gemv_shape_ok(I[j], M[j], N, T)) return 0;
+    const int path = group_path(I, M, n, N, K, T);
+    if (path < 0) return 0;
+    if (path == 1) return strip_part_floats(I, M, n, N, K, T) * (int64_t)sizeof(float);
     const Plan p = make_plan(I, M, n, N, pass_tokens(T));
     return p.part_total * (int64_t)sizeof(float);
 }
@@ -749,7 +813,7 @@ int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, 
 // (0 in *waves when the decode kernel does not take them).
 void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax) {
     *waves = *row_tiles_per_wave = *grid = *kmax = 0;
-    if (!gemv_shape_ok(I, M, N, T)) return;
+    if (group_path(&I, &M, 1, N, 16, T) != 0) return;
     const Plan p = make_plan(&I, &M, 1, N, pass_tokens(T));
     *waves = p.waves;
     *row_tiles_per_wave = p.R;

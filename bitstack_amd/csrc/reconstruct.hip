@@ -84,12 +84,22 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
         if (row_begin + wave * 16 < row_end) load_block(i0, min(row_begin + wave * 16 + lm, M - 1), b_cur, sw_cur);
 
-        for (int i = 0; i < ib; i++) {
-            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (sr < K)
-                v = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
+        // four blocks at a time, so that their loads are in flight together
+        for (int q0 = 0; q0 < ib; q0 += 4) {
+            half8_t v[4];
 #pragma unroll
-            for (int e = 0; e < 8; e++) vl[i * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[e];
+            for (int k = 0; k < 4; k++) {
+                const int i = min(q0 + k, ib - 1);
+                v[k] = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
+                if (sr < K) v[k] = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + 8 * sp);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if (q0 + k < ib) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vl[(q0 + k) * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[k][e];
+                }
+            }
         }
         __syncthreads();
 

@@ -93,8 +93,11 @@ int64_t bs_workspace_bytes(int I, int M, int N, int K, int T);
  * reconstruct_and_forward_triton + fused_reconstruct_and_forward_kernel
  * (bitstack/utils/inference_utils.py:171-284).
  *
- * T <= 8 runs the packed-sign GEMV (signs contracted on MFMA against
- * vt_i o x, scaled by u_i, all blocks in one pass); larger T rebuilds the
+ * T <= 4 runs the packed-sign GEMV (signs contracted on MFMA against
+ * vt_i o x, scaled by u_i, all blocks in one pass; N % 512 == 0); 5 <= T <= 32
+ * the strip kernel (16 x 16 patches of the weight rebuilt in registers and
+ * multiplied by x at once, the weight never stored; N % 128 == 0; when it does
+ * not take the shape, T <= 8 is two GEMV passes); larger T rebuilds the
  * weight once into `workspace` and runs a dense MFMA GEMM.  Requires
  * N % 8 == 0.  `workspace` must hold bs_workspace_bytes(...) bytes, 256-byte
  * aligned; its contents on entry do not matter and it may be reused by the
@@ -108,8 +111,9 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * Introspection for benchmarks and tests: which decode kernel instantiation
  * (waves per workgroup, 16-row tiles per wave), how many workgroups and how
  * many partial sums per row and block bs_forward would use for these
- * dimensions; *waves == 0 means the decode kernel does not take them (more
- * than 8 tokens, N not a multiple of 512).  No counterpart in the reference
+ * dimensions; *waves == 0 means the decode kernel does not run them (the
+ * strip kernel or the dense path does: more than 4 tokens with N % 128 == 0,
+ * more than 8 tokens, N not a multiple of 512).  No counterpart in the reference
  * (Triton picks its configuration by autotuning,
  * bitstack/utils/inference_utils.py:8-39).
  */
@@ -127,7 +131,7 @@ int bs_linear_f16(const void *x, const void *w, const void *bias, void *y,
 
 /*
  * ---- decode step: several matrices per launch, fused epilogues -----------
- * One decode forward (T <= 8 tokens) of up to 4 compressed matrices that read
+ * One decode forward (T <= 32 tokens; more than 8 need N % 128 == 0) of up to 4 compressed matrices that read
  * the same x, in one kernel pair: what q_proj/k_proj/v_proj (or gate_proj/
  * up_proj) of a decoder layer do with three (two) BitStackLinear.forward calls,
  * bitstack/modules/BitStackLinear.py:88-157, each as in bs_forward.  All share

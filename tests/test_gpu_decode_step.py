@@ -46,7 +46,8 @@ def make_group(shapes, N, T, seed, bias=False):
 
 GROUP_CASES = [([(3, 512), (5, 128), (2, 128)], 512, 1), ([(3, 4096), (5, 1024), (2, 1024)], 4096, 1),
                ([(2, 1024), (4, 256)], 1024, 2), ([(1, 300), (2, 77), (3, 64), (1, 512)], 1536, 3),
-               ([(2, 512), (3, 256)], 1024, 4), ([(2, 512), (1, 256)], 512, 5), ([(2, 256), (2, 256)], 1024, 8)]
+               ([(2, 512), (3, 256)], 1024, 4), ([(2, 512), (1, 256)], 512, 5), ([(2, 256), (2, 256)], 1024, 8),
+               ([(2, 300), (3, 77), (1, 64)], 1536, 9), ([(3, 1024), (2, 256)], 4096, 16), ([(2, 200), (2, 200)], 384, 32)]
 
 
 @pytest.mark.parametrize("shapes,N,T", GROUP_CASES)
@@ -64,7 +65,7 @@ def test_group_forward_side_by_side(shapes, N, T):
         off += M
 
 
-@pytest.mark.parametrize("I,M,N,T", [(3, 512, 1024, 1), (2, 4096, 4096, 1), (2, 256, 512, 6)])
+@pytest.mark.parametrize("I,M,N,T", [(3, 512, 1024, 1), (2, 4096, 4096, 1), (2, 256, 512, 6), (2, 300, 640, 12)])
 def test_group_forward_residual(I, M, N, T):
     print(f"group residual I={I} M={M} N={N} T={T}", flush=True)
     grp, x, refs = make_group([(I, M)], N, T, seed=21)
@@ -75,7 +76,7 @@ def test_group_forward_residual(I, M, N, T):
     assert np.array_equal(y, (res.float() + plain.float()).half().numpy())        # exactly the fp16 add of the fp16 result
 
 
-@pytest.mark.parametrize("I0,I1,M,N,T", [(3, 2, 1024, 512, 1), (2, 4, 14336, 4096, 1), (2, 2, 512, 1024, 7)])
+@pytest.mark.parametrize("I0,I1,M,N,T", [(3, 2, 1024, 512, 1), (2, 4, 14336, 4096, 1), (2, 2, 512, 1024, 7), (2, 3, 1024, 2048, 24)])
 def test_group_forward_swiglu(I0, I1, M, N, T):
     print(f"group swiglu I={I0},{I1} M={M} N={N} T={T}", flush=True)
     grp, x, refs = make_group([(I0, M), (I1, M)], N, T, seed=31)
@@ -93,7 +94,7 @@ def test_group_forward_swiglu(I0, I1, M, N, T):
 def test_group_rejects_what_the_decode_kernel_does_not_take():
     grp, x, _ = make_group([(1, 64), (1, 64)], 512, 1, seed=1)
     with pytest.raises(RuntimeError):
-        IU.bitstack_forward_group_hip(grp, torch.zeros(9, 512, dtype=torch.float16, device=dev()))    # more than 8 tokens
+        IU.bitstack_forward_group_hip(grp, torch.zeros(33, 512, dtype=torch.float16, device=dev()))   # more than 32 tokens
     grp2, _, _ = make_group([(1, 64), (1, 128)], 512, 1, seed=1)
     with pytest.raises(RuntimeError):
         IU.bitstack_forward_group_hip(grp2, x.to(dev()), _lib.EPI_SWIGLU)                               # unequal M
@@ -262,6 +263,7 @@ def test_decoder_round_trips_through_a_checkpoint(tmp_path):
                                               ([(2, 4096), (3, 1024), (1, 1024)], 4096, 1, "none"),
                                               ([(2, 1024), (3, 1024)], 2048, 1, "swiglu"),
                                               ([(2, 256), (1, 256)], 512, 5, "swiglu"),
+                                              ([(2, 512), (3, 128)], 1024, 20, "none"),
                                               ([(2, 300)], 1536, 3, "none")])
 def test_group_forward_with_input_rms(shapes, N, T, mode):
     """bs_forward_group_rms: the RMSNorm in front of the matrices without a launch of its own.  The

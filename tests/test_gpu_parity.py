@@ -163,6 +163,32 @@ def test_forward_odd_shapes_take_the_rebuild_path(I, M, N, T):
     assert_close(y, l0, "vs level-0 order")
 
 
+# 5..32 tokens: weight patches rebuilt in registers and multiplied at once (N a multiple of 128)
+STRIP_CASES = [(1, 16, 128, 5, 16), (3, 100, 384, 9, 16), (2, 65, 1152, 17, 7), (4, 1000, 2048, 32, 16),
+               (20, 64, 256, 6, 16), (2, 4096, 4096, 32, 16), (3, 14336, 4096, 8, 16), (2, 1024, 14336, 16, 16),
+               (36, 130, 128, 12, 3)]
+
+
+@pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)
+def test_forward_few_dozen_tokens_matches_oracle(I, M, N, T, K):
+    print(f"forward strips I={I} M={M} N={N} T={T} K={K}", flush=True)
+    assert _lib.decode_plan(I, M, N, K, T)[0] == 0        # not the decode kernel
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=3 * I + T, signed_factors=True)
+    bias = (torch.randn(M, generator=torch.Generator().manual_seed(T)) * 0.05).half() if T % 2 else None
+    exact, l0 = oracle_refs(q, u, vt, x, bias)
+    qd, ud, vd, xd = q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())
+    y = IU.bitstack_forward_hip(qd, ud, vd, xd, None if bias is None else bias.to(dev())).cpu().numpy()
+    assert y.dtype == np.float16 and y.shape == (T, M)
+    assert_close(y, exact, "vs fp64")
+    if I <= 8:      # with more blocks the level-0 order's own fp16 sums are further from fp64 than the bound
+        assert_close(y, l0, "vs level-0 order")
+    # the same rounding points as rebuilding the fp16 weight and multiplying: only the order of the
+    # fp32 sums differs
+    w = IU.unpack_and_reconstruct_w_hip(qd, ud, vd)
+    dense = IU.linear_f16_hip(xd, w, None if bias is None else bias.to(dev())).cpu().numpy()
+    assert_close(y, dense, "vs rebuilt weight x dense kernel", 2e-3, 2e-4)
+
+
 PREFILL_CASES = [(2, 256, 512, 16), (8, 1024, 4096, 16), (4, 1024, 1024, 128), (2, 300, 1024, 100),
                  (8, 4096, 4096, 128), (2, 512, 1024, 512)]
 

@@ -94,7 +94,8 @@ def test_group_and_decode_step_validation(L):
     assert L.bs_forward_group_workspace_bytes(mats, 2, 500, 16, 1) == -2          # N % 8
     assert L.bs_forward_group_workspace_bytes(mats, 2, 520, 16, 1) == -2          # not a decode-kernel shape
     assert L.bs_forward_group_workspace_bytes(mats, 5, 512, 16, 1) == -2          # more than BS_MAX_GROUP
-    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 9) == -2          # more than 8 tokens
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 9) > 0            # 9..32 tokens: the strip kernel
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 33) == -2         # more than 32 tokens
     assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 17, 1) == -3
     assert L.bs_forward_group_workspace_bytes(nul, 2, 512, 16, 1) == -1
     big = 1 << 30
