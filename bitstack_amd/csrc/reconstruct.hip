@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
             for (int i = 0; i < ib; i++) {
                 if (i + 1 < ib) load_block(i0 + i + 1, row, b_nxt, sw_nxt);
                 else if (m0 + 64 < row_end) load_block(i0, min(m0 + 64 + lm, M - 1), b_nxt, sw_nxt);
-                const uint4_t swc = ~sw_cur;     // bit 1 means +1: make it a clear IEEE sign bit
+                const uint4_t swc = sw_cur;      // bit 1 means +1: the product enters negated, times -1.0f
                 const half_t *vb = vl + i * VBLOCK + aoff;
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                            acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                            acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
                         }
                     } else {
                         uint32_t t = *reinterpret_cast<const uint32_t *>(

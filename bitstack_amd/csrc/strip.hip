@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
                 if (i + 1 < I) load_block(i + 1, row, q, b_nxt, sw_nxt);
                 else if (q + 1 < ns) load_block(0, row, q + 1, b_nxt, sw_nxt);
                 else if (m0 + 64 < row_end) load_block(0, min(m0 + 64 + lm, M - 1), 0, b_nxt, sw_nxt);
-                const uint4_t swc = ~sw_cur;        // bit 1 means +1: make it a clear IEEE sign bit
+                const uint4_t swc = sw_cur;         // bit 1 means +1: the product enters negated, times -1.0f
                 const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                        acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                        acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
                     }
                 }
                 b_cur = b_nxt;
