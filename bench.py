@@ -21,7 +21,7 @@ Extra objects on the same JSON line:
                 region (events recorded on the stream the kernels run on).
   cpu_baseline  the reference's CPU path (level 0) restated in torch-CPU ops,
                 timed on this host on one pass of the same sweep.
-  t4, prefill   the same sweep at 4 tokens, and the prefill configuration
+  t4, t16, prefill   the same sweep at 4 and at 16 tokens, and the prefill configuration
                 (I = 8, T in {16, 128, 512, 2048}) as useful TFLOP/s.
   decode_8b     tokens/s of a random-init Llama-3.1-8B-shape decode loop built
                 around the same forward (batch 1, 256 greedy tokens).
@@ -52,6 +52,7 @@ def parse():
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
     ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
+    ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..32)")
     ap.add_argument("--layer", default="14336x4096x16x1",
                     help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
@@ -104,8 +105,9 @@ def cpu_baseline(layers_cpu):
 
 def e2e_decode_70b(torch, dev, batch=8, prompt_len=16, new_tokens=64):
     """Random-init Llama-3.1-70B-shape decode, `batch` sequences in lock step (every
-    linear sees 8 tokens: two passes of four through the decode kernel), about 30 GB
-    of weights.  The prompt is fed token by token (prefill is not what is measured)."""
+    linear sees `batch` tokens: from five on that is the strip kernel, weight patches
+    rebuilt in registers and multiplied at once), about 30 GB of weights.  The prompt
+    is fed token by token (prefill is not what is measured)."""
     from bitstack_amd.utils.llama_decode import LLAMA_70B, SyntheticLlamaDecoder, synthetic_compression_config
     cfg, total = synthetic_compression_config(LLAMA_70B, 30e9, lo=1, hi=8)
     model = SyntheticLlamaDecoder(LLAMA_70B, cfg, prompt_len + new_tokens + 8, dev, batch=batch)
@@ -300,7 +302,7 @@ def main():
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
         return
     if a.only == "decode_70b":
-        print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev)}))
+        print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev, batch=a.batch)}))
         return
     if a.only == "prefill":
         print(json.dumps({"prefill": prefill_side([])}))
@@ -375,6 +377,16 @@ def main():
         detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 4, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l4, per4)]
         del l4
+        # ------------------------------------------------------------ T = 16 sweep (strip kernel: batched decode)
+        l16 = build_sweep(16)
+        _, per16 = time_sweep(l16, max(3, a.steps // 2), 1, per_layer_events=True)
+        b16 = sum(L.bytes for L in l16)
+        t16 = sum(per16) * 1e-3
+        out["t16"] = {"GBps": round(b16 / t16 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b16 / t16 / 1e9 / HBM_PEAK_GBS, 2),
+                      "kernel": "strip_forward_kernel<1> + gemv_reduce_kernel"}
+        detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 16, "bytes": L.bytes, "us": round(ms * 1e3, 2),
+                    "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l16, per16)]
+        del l16
         # ------------------------------------------------------------ prefill (useful flops)
         pre = prefill_side(detail)
         out["prefill"] = pre
