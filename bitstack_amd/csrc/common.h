@@ -67,8 +67,9 @@ int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *cons
                          int64_t workspace_bytes, hipStream_t s);
 // strip kernel (strip.hip): partial sums part[strip, t, m] of x . w^T with w rebuilt in registers
 int bs_strip_partials(int I, int M, int N, int K, int T);
-int bs_launch_strip_partials(const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-                             float *part, int I, int M, int N, int K, int T, hipStream_t s);
+int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
+                          const int *I, const int *M, float *const *part, float *ssq, const half_t *x,
+                          int N, int K, int T, hipStream_t s);
 // decode-step kernels around the linears (decode_step.hip)
 int bs_launch_argmax(const half_t *x, int64_t *out, int B, int V, hipStream_t s);
 int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s);

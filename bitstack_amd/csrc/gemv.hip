@@ -440,6 +440,10 @@ struct RedGroup {
     const half_t *xin;
     int n_in;
     float eps;
+    // the same scale from ready-made partial sums of squares, ssq[g * T + t] for g < ssq_n
+    // (written by the strip kernel); takes precedence over xin
+    const float *ssq;
+    int ssq_n;
 };
 
 // Sum of the partials of output m of one matrix that this thread's slice covers.
@@ -511,20 +515,25 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     }
     float scale = 1.f;
     __shared__ float ssq[RED_OUT * RED_SL / 64];
-    if (grp.xin) {                               // sum of squares of this token's input row, every workgroup for itself
-        const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
+    const bool scaled = grp.xin || grp.ssq;
+    if (scaled) {                                // sum of squares of this token's input row, every workgroup for itself
         float q = 0.f;
-        for (int c = threadIdx.x * 8; c < grp.n_in; c += RED_OUT * RED_SL * 8) {
-            const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
+        if (grp.ssq) {
+            for (int c = threadIdx.x; c < grp.ssq_n; c += RED_OUT * RED_SL) q += grp.ssq[c * T + t];
+        } else {
+            const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
+            for (int c = threadIdx.x * 8; c < grp.n_in; c += RED_OUT * RED_SL * 8) {
+                const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
 #pragma unroll
-            for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+                for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+            }
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o, 64);
         if ((threadIdx.x & 63) == 0) ssq[threadIdx.x >> 6] = q;
     }
     __syncthreads();
-    if (grp.xin) {
+    if (scaled) {
         float q = 0.f;
 #pragma unroll
         for (int w = 0; w < RED_OUT * RED_SL / 64; w++) q += ssq[w];
@@ -686,13 +695,13 @@ int group_path(const int *I, const int *M, int n, int N, int K, int T) {
     return -1;
 }
 int64_t strip_part_floats(const int *I, const int *M, int n, int N, int K, int T) {
-    int64_t total = 0;
+    int64_t total = (int64_t)bs_strip_partials(I[0], M[0], N, K, T) * T;      // sums of squares of x per strip group
     for (int j = 0; j < n; j++) total += (int64_t)bs_strip_partials(I[j], M[j], N, K, T) * T * M[j];
     return total;
 }
 
-// Strip path: one launch per matrix writes part[strip, t, m]; the reduce kernel reads that
-// as "one partial per block" with the strips in the place of the blocks.
+// Strip path: one launch writes part[strip group, t, m] of every matrix; the reduce kernel
+// reads that as "one partial per block" with the strip groups in the place of the blocks.
 int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T, int mode, const half_t *residual,
                         half_t *y, bool input_rms, float eps, void *workspace, int64_t workspace_bytes, hipStream_t s) {
     if (!workspace || workspace_bytes < strip_part_floats(a.I, a.M, a.n, N, K, T) * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
@@ -700,20 +709,25 @@ int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T
     RedGroup r;
     r.n = a.n;
     r.mode = mode;
-    r.xin = input_rms ? x : nullptr;
+    r.xin = nullptr;
     r.n_in = N;
     r.eps = eps;
+    float *parts[GEMV_MAX_GROUP];
     int ldy = 0, blocks = 0;
     int64_t off = 0;
     for (int j = 0; j < a.n; j++) {
-        const int st = bs_launch_strip_partials(a.packed[j], a.u[j], a.vt[j], x, part + off, a.I[j], a.M[j], N, K, T, s);
-        if (st != BS_OK) return st;
         const int groups = bs_strip_partials(a.I[j], a.M[j], N, K, T);
+        parts[j] = part + off;
         r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], (int)bs_cdiv(a.M[j], RED_OUT), 1, ldy, blocks, Split{1, 0}};
         off += (int64_t)groups * T * a.M[j];
         ldy += a.M[j];
         if (mode != EPI_SWIGLU || j == 0) blocks += T * (int)bs_cdiv(a.M[j], RED_OUT);
     }
+    r.ssq = input_rms ? part + off : nullptr;
+    r.ssq_n = r.m[0].I;
+    const int st = bs_launch_strip_group(a.n, a.packed, a.u, a.vt, a.I, a.M, parts, input_rms ? part + off : nullptr,
+                                         x, N, K, T, s);
+    if (st != BS_OK) return st;
     if (mode == EPI_SWIGLU) ldy = a.M[0];
     for (int j = a.n; j < GEMV_MAX_GROUP; j++) r.m[j] = r.m[0];
     gemv_reduce_kernel<<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, RED_OUT, 1);
@@ -754,6 +768,8 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
     r.xin = nullptr;
     r.n_in = N;
     r.eps = eps;
+    r.ssq = nullptr;
+    r.ssq_n = 0;
     int y_off = 0, blocks = 0;
     for (int j = 0; j < a.n; j++) {
         g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],

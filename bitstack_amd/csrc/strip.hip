@@ -31,30 +31,58 @@ constexpr int VBLOCK = SF_COLS * VSTRIDE + (SF_COLS / 8) * VGROUP_PAD;   // halv
 // their vt slices are staged together, and per 16-row step the partial y of all of them
 // is added up in registers, so scratch holds one partial per GROUP of strips and a lane
 // reads sg * 16 consecutive sign bytes of its row.
+// Up to four matrices that read the same x share a launch (q/k/v, gate/up): the grid is cut
+// into one run of slots per matrix, each with its own strips per workgroup and row split.
+constexpr int STRIP_MAX_GROUP = 4;
+struct StripMat {
+    const uint8_t *packed;
+    const half_t *u, *vt;
+    float *part;
+    int I, M, sg, rows_per_wg, row_groups, first_slot;
+};
+struct StripGroup {
+    StripMat m[STRIP_MAX_GROUP];
+    int n;
+    float *ssq;     // [strip groups of matrix 0][T]: sum of x^2 over the group's columns (for an RMS scale), or null
+};
+
 template <int TT>
 __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
-    const uint8_t *__restrict__ packed, const half_t *__restrict__ u, const half_t *__restrict__ vt,
-    const half_t *__restrict__ x, float *__restrict__ part, int I, int M, int N, int K, int T, int sg,
-    int rows_per_wg) {
+    const StripGroup grp, const half_t *__restrict__ x, int N, int K, int T) {
     extern __shared__ __attribute__((aligned(16))) half_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 15, g = lane >> 4;
+    // Workgroups are dealt round-robin to the 8 XCDs.  Every matrix owns a run of block
+    // indices that starts at a multiple of 8, so each XCD gets an eighth of every matrix
+    // (their slots differ in work).  Within a matrix the slot order is (128-byte line of
+    // sign bytes, row group, strip group within the line) in contiguous runs per XCD: the
+    // 8 / sg groups that share a line meet in one L2.  Strip groups are padded to whole
+    // lines and the slots to a multiple of 8; slots beyond the last strip idle.
+    StripMat mat = grp.m[0];
+    bool first_matrix = true;
+    int slots = grp.n > 1 ? grp.m[1].first_slot : (int)gridDim.x;
+#pragma unroll
+    for (int j = 1; j < STRIP_MAX_GROUP; j++)
+        if (j < grp.n && (int)blockIdx.x >= grp.m[j].first_slot) {
+            mat = grp.m[j];
+            first_matrix = false;
+            slots = (j + 1 < grp.n ? grp.m[j + 1].first_slot : (int)gridDim.x) - mat.first_slot;
+        }
+    const int local = (int)blockIdx.x - mat.first_slot;
+    const int slot = (local & 7) * (slots >> 3) + (local >> 3);
+    const uint8_t *__restrict__ packed = mat.packed;
+    const half_t *__restrict__ u = mat.u;
+    const half_t *__restrict__ vt = mat.vt;
+    float *__restrict__ part = mat.part;
+    const int I = mat.I, M = mat.M, sg = mat.sg, rows_per_wg = mat.rows_per_wg;
     const int xstride = sg * SF_COLS + 8;           // halves per token row of the x image
     half_t *xl = lds;                               // [TT * 16][xstride]
     half_t *vl = lds + TT * 16 * xstride;           // [sg][I][VBLOCK]
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int lm = lane & 15, g = lane >> 4;
-    // Slot order (128-byte line of sign bytes, row group, strip group within the line),
-    // contiguous runs of slots per XCD: the 8 / sg groups that share a line meet in one L2.
-    // gridDim.x counts strip groups padded to whole lines; slots beyond the last strip idle.
     int group, row_begin;
     {
-        const int per_line = 8 / sg;
-        const int nb = gridDim.x * gridDim.y, lin = blockIdx.x + gridDim.x * blockIdx.y;
-        const int xcd = lin & 7, loc = lin >> 3, base = nb >> 3, rem = nb & 7;
-        const int v = xcd * base + min(xcd, rem) + loc;
-        const int rest = v / per_line;
-        group = (rest / (int)gridDim.y) * per_line + v % per_line;
-        row_begin = (rest % (int)gridDim.y) * rows_per_wg;
+        const int per_line = 8 / sg, rest = slot / per_line;
+        group = (rest / mat.row_groups) * per_line + slot % per_line;
+        row_begin = (rest % mat.row_groups) * rows_per_wg;
     }
     const int strips = N / SF_COLS;
     const int s_begin = group * sg;
@@ -109,6 +137,23 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
         }
     }
     __syncthreads();
+
+    // sum of squares of every token over this group's columns, once per strip group
+    if (grp.ssq && first_matrix && row_begin == 0) {
+        const int t = tid >> 3, sub = tid & 7;
+        float q = 0.f;
+        if (t < TT * 16) {
+            for (int c = sub * 8; c < ns * SF_COLS; c += 64) {
+                const half8_t v = *reinterpret_cast<const half8_t *>(xl + t * xstride + c);
+#pragma unroll
+                for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+            }
+        }
+        q += __shfl_xor(q, 1, 64);
+        q += __shfl_xor(q, 2, 64);
+        q += __shfl_xor(q, 4, 64);
+        if (sub == 0 && t < T) grp.ssq[group * T + t] = q;
+    }
 
     // this lane's x fragments: token lm of a tile, columns 32 (s / 2) + 8 g + 4 (s % 2) .. + 3 of patch s
     const half_t *xfrag = xl + lm * xstride + 8 * g;
@@ -211,13 +256,11 @@ StripPlan make_strip_plan(int I, int M, int N, int T) {
 }
 
 template <int TT>
-int launch_tt(const StripPlan &p, const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-              float *part, int I, int M, int N, int K, int T, hipStream_t s) {
+int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
     static size_t granted[BS_MAX_DEVICES] = {};
-    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT>, p.lds, granted);
+    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT>, lds, granted);
     if (st != BS_OK) return st;
-    dim3 grid(p.gx, p.row_groups);
-    strip_forward_kernel<TT><<<grid, 256, p.lds, s>>>(packed, u, vt, x, part, I, M, N, K, T, p.sg, p.rows_per_wg);
+    strip_forward_kernel<TT><<<grid, 256, lds, s>>>(grp, x, N, K, T);
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
@@ -234,14 +277,25 @@ int bs_strip_partials(int I, int M, int N, int K, int T) {
     return p.groups <= 1024 ? p.groups : 0;
 }
 
-// part[group of strips, t, m]: bs_strip_partials x T x M floats
-int bs_launch_strip_partials(const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
-                             float *part, int I, int M, int N, int K, int T, hipStream_t s) {
-    if (bs_strip_partials(I, M, N, K, T) == 0) return BS_ERR_SHAPE;
-    if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(u, 8) || !bs_aligned(x, 16)) return BS_ERR_SHAPE;
-    const StripPlan p = make_strip_plan(I, M, N, T);
-    switch (p.tt) {
-        case 1: return launch_tt<1>(p, packed, u, vt, x, part, I, M, N, K, T, s);
-        default: return launch_tt<2>(p, packed, u, vt, x, part, I, M, N, K, T, s);
+// One launch for n <= 4 matrices that read x: part[j] receives [bs_strip_partials(j), T, M[j]]
+// floats; ssq (may be null) receives [bs_strip_partials(0), T] sums of squares of x.
+int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
+                          const int *I, const int *M, float *const *part, float *ssq, const half_t *x,
+                          int N, int K, int T, hipStream_t s) {
+    if (n < 1 || n > STRIP_MAX_GROUP || !bs_aligned(x, 16)) return BS_ERR_SHAPE;
+    StripGroup grp;
+    grp.n = n;
+    grp.ssq = ssq;
+    size_t lds = 0;
+    int slots = 0;
+    for (int j = 0; j < n; j++) {
+        if (bs_strip_partials(I[j], M[j], N, K, T) == 0) return BS_ERR_SHAPE;
+        if (!bs_aligned(packed[j], 16) || !bs_aligned(vt[j], 16) || !bs_aligned(u[j], 8)) return BS_ERR_SHAPE;
+        const StripPlan p = make_strip_plan(I[j], M[j], N, T);
+        grp.m[j] = StripMat{packed[j], u[j], vt[j], part[j], I[j], M[j], p.sg, p.rows_per_wg, p.row_groups, slots};
+        slots += (int)bs_cdiv(p.gx * p.row_groups, 8) * 8;
+        if (p.lds > lds) lds = p.lds;
     }
+    for (int j = n; j < STRIP_MAX_GROUP; j++) grp.m[j] = grp.m[0];
+    return token_tiles(T) == 1 ? launch_tt<1>(grp, slots, lds, x, N, K, T, s) : launch_tt<2>(grp, slots, lds, x, N, K, T, s);
 }

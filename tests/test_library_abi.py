@@ -80,9 +80,13 @@ def test_workspace_bytes(L):
     assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2
     assert L.bs_workspace_bytes(2, 64, 72, 16, 1) == ((64 * 72 * 2 + 255) // 256) * 256
     # decode keeps fp32 partial row sums: a multiple of T * M * 4, far below the weight
-    for T in (1, 4, 8):
+    for T in (1, 4):
         b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
         assert b > 0 and b % (T * 4096 * 4) == 0 and b < 4096 * 4096 * 2
+    # 5..32 tokens: partial sums per group of strips (plus the groups' sums of squares of x)
+    for T in (8, 32):
+        b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
+        assert T * 4096 * 4 <= b <= 32 * (T * 4096 * 4 + T * 4) + 256
 
 
 def test_group_and_decode_step_validation(L):
