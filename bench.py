@@ -53,6 +53,7 @@ def parse():
     ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..32)")
+    ap.add_argument("--prompt-len", type=int, default=2048, help="prompt tokens per sequence of --only decode_70b")
     ap.add_argument("--layer", default="14336x4096x16x1",
                     help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
@@ -103,19 +104,27 @@ def cpu_baseline(layers_cpu):
             "seconds": round(tot_t, 2)}
 
 
-def e2e_decode_70b(torch, dev, batch=8, prompt_len=16, new_tokens=64):
-    """Random-init Llama-3.1-70B-shape decode, `batch` sequences in lock step (every
-    linear sees `batch` tokens: from five on that is the strip kernel, weight patches
-    rebuilt in registers and multiplied at once), about 30 GB of weights.  The prompt
-    is fed token by token (prefill is not what is measured)."""
+def e2e_decode_70b(torch, dev, batch=8, prompt_len=2048, new_tokens=128):
+    """Random-init Llama-3.1-70B-shape model, about 30 GB of weights, `batch` sequences in
+    lock step: the prompt in one pass (every linear sees batch * prompt_len tokens: rebuild +
+    dense kernels; causal attention is torch's), then greedy decode (every linear sees `batch`
+    tokens: from five on that is the strip kernel, weight patches rebuilt in registers and
+    multiplied at once), one HIP-graph replay per step."""
     from bitstack_amd.utils.llama_decode import LLAMA_70B, SyntheticLlamaDecoder, synthetic_compression_config
     cfg, total = synthetic_compression_config(LLAMA_70B, 30e9, lo=1, hi=8)
     model = SyntheticLlamaDecoder(LLAMA_70B, cfg, prompt_len + new_tokens + 8, dev, batch=batch)
     prompt = torch.randint(0, LLAMA_70B.vocab, (batch, prompt_len), generator=torch.Generator().manual_seed(0)).to(dev)
+    model.prefill(prompt[:, :min(prompt_len, 64)])          # warm-up: workspaces, kernel attributes
+    model.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.prefill(prompt)
+    torch.cuda.synchronize()
+    dt_prefill = time.perf_counter() - t0
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        model.prefill_positions(prompt, fused=True)
+        model.step_fused()                                  # warm-up of the decode step outside capture
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
@@ -129,11 +138,17 @@ def e2e_decode_70b(torch, dev, batch=8, prompt_len=16, new_tokens=64):
     dt = time.perf_counter() - t0
     wbytes = model.weight_bytes()
     blocks = list(cfg.values())
+    s = LLAMA_70B
+    per_tok = 2.0 * sum(m * n for (m, n) in (s.proj_shape(p) for p in
+                        ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
+                         "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj"))) * s.layers
     return {"tok_s": round(batch * new_tokens / dt, 1), "ms_per_step": round(dt / new_tokens * 1e3, 3), "batch": batch,
+            "prefill_s": round(dt_prefill, 3), "prefill_tok_s": round(batch * prompt_len / dt_prefill, 1),
+            "prefill_linear_tflops": round(per_tok * batch * prompt_len / dt_prefill / 1e12, 1),
             "weight_GB": round(wbytes / 1e9, 2), "blocks_per_linear_mean": round(sum(blocks) / len(blocks), 2),
             "hbm_roofline_tok_s": round(batch * 8e12 / wbytes, 1),
-            "config": f"80 layers, hidden 8192, inter 28672, 64Q/8KV, vocab 128256, batch {batch}, {prompt_len}-token prompt, "
-                      f"{new_tokens} greedy tokens per sequence, fused step, one HIP-graph replay per step"}
+            "config": f"80 layers, hidden 8192, inter 28672, 64Q/8KV, vocab 128256, batch {batch}, {prompt_len}-token prompt in one "
+                      f"pass, {new_tokens} greedy tokens per sequence, fused step, one HIP-graph replay per step"}
 
 
 def e2e_decode(torch, dev, prompt_len=128, new_tokens=256):
@@ -302,7 +317,7 @@ def main():
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
         return
     if a.only == "decode_70b":
-        print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev, batch=a.batch)}))
+        print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev, batch=a.batch, prompt_len=a.prompt_len)}))
         return
     if a.only == "prefill":
         print(json.dumps({"prefill": prefill_side([])}))

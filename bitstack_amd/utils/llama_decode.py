@@ -300,6 +300,43 @@ class SyntheticLlamaDecoder:
         argmax_hip(self.logits, out=self.token)
         self.pos.add_(1)
 
+    @torch.no_grad()
+    def prefill(self, prompt: torch.Tensor):
+        """The whole prompt [batch, len] in one pass: every linear sees batch * len tokens (the
+        library's rebuild + dense path), causal attention and RoPE are torch ops, the KV cache
+        is filled for positions 0 .. len - 1, and self.token becomes the greedy token after
+        the prompt.  Decode continues from there with step() or step_fused()."""
+        s, B = self.s, self.batch
+        prompt = prompt.view(1, -1).expand(B, -1) if prompt.dim() == 1 else prompt
+        n = prompt.shape[1]
+        if n < 1 or n > self.max_len:
+            raise ValueError("prompt length must be in 1..max_len")
+        d = s.head_dim
+        x = self.embed.index_select(0, prompt.reshape(-1))                # [B * n, h]
+        cos, sin = self.cos[:n].view(1, 1, n, d // 2), self.sin[:n].view(1, 1, n, d // 2)
+        for L in range(s.layers):
+            lin = self.lin[L]
+            hn = rmsnorm_hip(x, self.norm_w[L, 0], s.rms_eps)
+            q = lin["self_attn.q_proj"](hn).view(B, n, s.heads, d).transpose(1, 2)
+            k = lin["self_attn.k_proj"](hn).view(B, n, s.kv_heads, d).transpose(1, 2)
+            v = lin["self_attn.v_proj"](hn).view(B, n, s.kv_heads, d).transpose(1, 2)
+            q, k = self._rope(q, cos, sin), self._rope(k, cos, sin)
+            self.kcache[L][:, :, :n].copy_(k)
+            self.vcache[L][:, :, :n].copy_(v)
+            ctx = torch.empty(B, n, s.hidden, dtype=torch.float16, device=self.dev)
+            for b in range(B):                                            # one sequence at a time bounds the scratch
+                o = F.scaled_dot_product_attention(q[b:b + 1], k[b:b + 1], v[b:b + 1], is_causal=True, enable_gqa=True)
+                ctx[b].copy_(o[0].transpose(0, 1).reshape(n, s.hidden))
+            x = x + lin["self_attn.o_proj"](ctx.view(B * n, s.hidden))
+            hn = rmsnorm_hip(x, self.norm_w[L, 1], s.rms_eps)
+            act = F.silu(lin["mlp.gate_proj"](hn))
+            act.mul_(lin["mlp.up_proj"](hn))
+            x = x + lin["mlp.down_proj"](act)
+        last = x.view(B, n, s.hidden)[:, -1].contiguous()
+        self.logits = F.linear(rmsnorm_hip(last, self.final_norm, s.rms_eps), self.lm_head)
+        self.token.copy_(self.logits.argmax(-1))
+        self.pos.fill_(n)
+
     def prefill_positions(self, prompt: torch.Tensor, fused=False):
         """Feed a prompt token by token (the measurement is about decode).  `prompt`
         is [len] (the same for every sequence) or [batch, len]."""

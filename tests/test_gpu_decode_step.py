@@ -208,6 +208,43 @@ def test_fused_step_matches_torch_step_and_float64_decoder(batch):
     assert_close(b.kcache.float().cpu().numpy(), a.kcache.float().cpu().numpy(), "k cache fused vs torch", 1e-2, 2e-3)
 
 
+@pytest.mark.parametrize("batch,n", [(1, 9), (3, 17)])
+def test_one_pass_prefill_matches_token_by_token_and_float64_decoder(batch, n):
+    """prefill(): all prompt positions at once (rebuild + dense kernels, causal attention in
+    torch) leaves the same logits, next token and KV cache as feeding the prompt position by
+    position, and decode continues from it."""
+    print(f"one-pass prefill batch={batch} n={n}", flush=True)
+    cfg = small_config()
+    a = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=6, batch=batch)
+    b = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=6, batch=batch)
+    with torch.no_grad():
+        for m in (a, b):
+            g = torch.Generator(device=dev()).manual_seed(3)
+            m.norm_w.copy_(1 + 0.2 * torch.randn(m.norm_w.shape, device=dev(), generator=g))
+            m.embed.mul_(30.0)
+    prompt = torch.randint(0, SMALL.vocab, (batch, n), generator=torch.Generator().manual_seed(2)).to(dev())
+    a.prefill_positions(prompt, fused=True)
+    b.prefill(prompt)
+    assert int(b.pos) == n == int(a.pos)
+    assert_close(b.logits.float().cpu().numpy(), a.logits.float().cpu().numpy(), "logits after the prompt", 2e-2, 4e-3)
+    assert_close(b.kcache[:, :, :, :n].float().cpu().numpy(), a.kcache[:, :, :, :n].float().cpu().numpy(), "k cache", 1e-2, 2e-3)
+    assert_close(b.vcache[:, :, :, :n].float().cpu().numpy(), a.vcache[:, :, :, :n].float().cpu().numpy(), "v cache", 1e-2, 2e-3)
+    assert float(b.kcache[:, :, :, n:].abs().max()) == 0.0
+    w = dense_weights(a)
+    for s_ in range(batch):
+        orc = LO.LlamaOracle(w, SMALL.layers, SMALL.heads, SMALL.kv_heads, SMALL.head_dim, SMALL.rope_theta, SMALL.rms_eps, 32)
+        for j in range(n):
+            want = orc.step(int(prompt[s_, j]))
+        assert_close(b.logits[s_].float().cpu().numpy(), want, f"prefill vs float64, seq {s_}", 2e-2, 4e-3)
+    # decode goes on from the prefilled cache
+    b.token.copy_(a.token)
+    for _ in range(3):
+        a.step_fused()
+        b.step_fused()
+        assert_close(b.logits.float().cpu().numpy(), a.logits.float().cpu().numpy(), "decode after prefill", 2e-2, 4e-3)
+        b.token.copy_(a.token)
+
+
 def test_fused_step_replays_in_a_graph():
     cfg = small_config(1)
     m = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=2)
