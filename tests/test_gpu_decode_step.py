@@ -116,10 +116,12 @@ def test_rmsnorm(T, H):
     assert (y.float() - want.float()).abs().max() <= 2 * torch.finfo(torch.float16).eps * want.float().abs().max()
 
 
-@pytest.mark.parametrize("B,heads,kv", [(1, 32, 8), (3, 4, 2), (2, 8, 8)])
-def test_attention_decode_steps(B, heads, kv):
-    print(f"attention B={B} heads={heads} kv={kv}", flush=True)
-    d, max_len, steps = 128, 40, 37
+@pytest.mark.parametrize("B,heads,kv,max_len", [(1, 32, 8, 40), (3, 4, 2, 40), (2, 8, 8, 40), (2, 16, 2, 40), (1, 6, 2, 40),
+                                                # long caches: several query heads of a KV head per workgroup
+                                                (2, 16, 2, 1100), (1, 32, 8, 1024), (2, 4, 2, 2048), (1, 6, 2, 1500)])
+def test_attention_decode_steps(B, heads, kv, max_len):
+    print(f"attention B={B} heads={heads} kv={kv} max_len={max_len}", flush=True)
+    d, steps = 128, 37
     g = torch.Generator().manual_seed(heads)
     cos64, sin64 = LO.rope_tables(max_len, d, 500000.0)
     cos, sin = torch.from_numpy(cos64).half(), torch.from_numpy(sin64).half()
@@ -147,12 +149,49 @@ def test_attention_decode_steps(B, heads, kv):
     assert float(kc[:, :, steps:].abs().max()) == 0.0 and float(vc[:, :, steps:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("B,heads,kv,max_len,at", [(2, 16, 2, 2048, 1500), (1, 8, 4, 1024, 1023), (1, 32, 8, 4096, 3000),
+                                                   (1, 4, 1, 1200, 517)])
+def test_attention_decode_deep_in_a_long_cache(B, heads, kv, max_len, at):
+    """One step at position `at` of a cache already holding random rows."""
+    print(f"attention deep B={B} heads={heads} kv={kv} max_len={max_len} at={at}", flush=True)
+    d = 128
+    g = torch.Generator().manual_seed(at)
+    cos64, sin64 = LO.rope_tables(max_len, d, 500000.0)
+    cos, sin = torch.from_numpy(cos64).half(), torch.from_numpy(sin64).half()
+    kc = torch.zeros(B, kv, max_len, d, dtype=torch.float16)
+    vc = torch.zeros_like(kc)
+    kc[:, :, :at] = torch.randn(B, kv, at, d, generator=g).half()
+    vc[:, :, :at] = torch.randn(B, kv, at, d, generator=g).half()
+    kd, vd = kc.to(dev()), vc.to(dev())
+    qkv = torch.randn(B, (heads + 2 * kv) * d, generator=g).half()
+    pos = torch.tensor([at], dtype=torch.long, device=dev())
+    out = IU.attention_decode_hip(qkv.to(dev()), kd, vd, cos.to(dev()), sin.to(dev()), pos, heads, kv).cpu().numpy()
+    x = qkv.double().numpy()
+    c, s_ = cos[at].double().numpy(), sin[at].double().numpy()
+    for b in range(B):
+        q = LO.rope(x[b, :heads * d].reshape(heads, d), c, s_)
+        kref, vref = kc[b].double().numpy().copy(), vc[b].double().numpy().copy()
+        kref[:, at] = LO.rope(x[b, heads * d:(heads + kv) * d].reshape(kv, d), c, s_).astype(np.float16)
+        vref[:, at] = x[b, (heads + kv) * d:].reshape(kv, d)
+        want = LO.attention_decode(q, kref, vref, at + 1).reshape(-1)
+        assert_close(out[b], want, f"attention at {at} seq {b}", 1e-2, 2e-3)
+        assert_close(kd[b, :, at].cpu().numpy(), kref[:, at], "appended k", 2e-3, 5e-4)
+    if at + 1 < max_len:
+        assert float(kd[:, :, at + 1:].abs().max()) == 0.0
+
+
 def test_attention_position_outside_the_cache_writes_zeros_and_touches_nothing():
     kc = torch.zeros(1, 2, 8, 128, dtype=torch.float16, device=dev())
     vc = torch.zeros_like(kc)
     tab = torch.ones(8, 64, dtype=torch.float16, device=dev())
     qkv = torch.ones(1, 8 * 128, dtype=torch.float16, device=dev())
     out = IU.attention_decode_hip(qkv, kc, vc, tab, tab, torch.tensor([8], device=dev()), 4, 2)
+    assert float(out.abs().max()) == 0.0 and float(kc.abs().max()) == 0.0
+    # the same through the grouped-query kernel of long caches
+    kc = torch.zeros(1, 2, 1024, 128, dtype=torch.float16, device=dev())
+    vc = torch.zeros_like(kc)
+    tab = torch.ones(1024, 64, dtype=torch.float16, device=dev())
+    out = IU.attention_decode_hip(qkv, kc, vc, tab, tab, torch.tensor([1024], device=dev()), 4, 2)
     assert float(out.abs().max()) == 0.0 and float(kc.abs().max()) == 0.0
 
 
