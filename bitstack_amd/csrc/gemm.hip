@@ -24,7 +24,8 @@
 // rows are padded), global requests at 64 B per clock: with 64 x 64 per-wave tiles the
 // LDS time equals the MFMA time, which is what the larger tiles are for.  Measured dead
 // ends: 128 x 128 per-wave tiles with one wave per SIMD (nothing covers a wait), a
-// per-workgroup rotation of the k order (less sharing in L2), 16-wave workgroups.
+// per-workgroup rotation of the k order (less sharing in L2), 16-wave workgroups, requests
+// that write LDS directly (global_load_lds_dwordx4: same time per step).
 // 33..128 tokens use narrower workgroups of the same kernel (more workgroups for
 // the few token rows); up to 32 tokens: linear_skinny_kernel (below).
 #include "common.h"
