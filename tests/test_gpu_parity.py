@@ -153,14 +153,15 @@ def test_forward_decode_signed_factors_bias_and_small_rank(I, M, N, T, K):
     assert_close(y.cpu().numpy(), l0, "vs level-0 order")
 
 
-@pytest.mark.parametrize("I,M,N,T", [(2, 40, 72, 1), (3, 33, 200, 3), (2, 64, 520, 9), (1, 16, 8, 1)])
+@pytest.mark.parametrize("I,M,N,T", [(2, 40, 72, 1), (3, 33, 200, 3), (2, 64, 520, 9), (1, 16, 8, 1), (40, 64, 256, 12)])
 def test_forward_odd_shapes_take_the_rebuild_path(I, M, N, T):
     print(f"forward odd I={I} M={M} N={N} T={T}", flush=True)
     q, u, vt, x = synthetic_layer(M, N, I, T, seed=2)
     exact, l0 = oracle_refs(q, u, vt, x)
     y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())).cpu().numpy()
     assert_close(y, exact, "vs fp64")
-    assert_close(y, l0, "vs level-0 order")
+    if I <= 8:      # with more blocks the level-0 order's own fp16 sums are further from fp64 than the bound
+        assert_close(y, l0, "vs level-0 order")
 
 
 # 5..32 tokens: weight patches rebuilt in registers and multiplied at once (N a multiple of 128)
