@@ -453,26 +453,34 @@ struct RedGroup {
 // workgroup) are loaded all the same (the slots exist in the workspace) and masked, so
 // the loads of a batch never wait for one another.  (i, k) advance incrementally: no
 // division in the loop.
-__device__ __forceinline__ float slice_sum_any(const RedMat &r, int T, int t, int m, int ks, const int *nks) {
+template <int VEC>
+struct RedVec { typedef float type; };
+template <>
+struct RedVec<4> { typedef float4_t type; };
+
+// VEC consecutive outputs m .. m + VEC - 1 per thread (VEC = 4: one 16-byte load per partial)
+template <int VEC>
+__device__ __forceinline__ typename RedVec<VEC>::type slice_sum_any(const RedMat &r, int T, int t, int m, int ks, const int *nks) {
+    typedef typename RedVec<VEC>::type vec_t;
     const int total = r.I * r.kmax;
     const int64_t stride = (int64_t)T * r.M;
     const float *base = r.part + (int64_t)t * r.M + m;
-    float acc = 0.f;
+    vec_t acc = vec_t(0.f);
     int i = ks / r.kmax, k = ks - i * r.kmax;                  // slot ks
     for (int s0 = ks; s0 < total; s0 += 4 * RED_SL) {
-        float v[4];
+        vec_t v[4];
         bool ok[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const bool in = s0 + j * RED_SL < total;
             const int ic = in ? i : 0, kc = in ? k : 0;
             ok[j] = in && kc < nks[ic];
-            v[j] = base[(int64_t)(ic * r.kmax + kc) * stride];
+            v[j] = *reinterpret_cast<const vec_t *>(base + (int64_t)(ic * r.kmax + kc) * stride);
             k += RED_SL;
             while (k >= r.kmax) { k -= r.kmax; i++; }
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc += ok[j] ? v[j] : 0.f;
+        for (int j = 0; j < 4; j++) acc += ok[j] ? v[j] : vec_t(0.f);
     }
     return acc;
 }
@@ -485,10 +493,18 @@ __device__ __forceinline__ void count_partials(const RedMat &r, int rt, int n_ch
     }
 }
 
+__device__ __forceinline__ float vec_get(float v, int) { return v; }
+__device__ __forceinline__ float vec_get(const float4_t &v, int e) { return v[e]; }
+
+// A workgroup produces RED_OUT * VEC consecutive outputs of one token.  VEC = 4 needs every M a
+// multiple of 4 (16-byte partial loads; the outputs are still stored one by one).
+template <int VEC>
 __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
     const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy,
     int rows_per_tile, int n_chunks) {
-    __shared__ float red[2][RED_SL][RED_OUT];
+    typedef typename RedVec<VEC>::type vec_t;
+    constexpr int RUN = RED_OUT * VEC;           // outputs per workgroup
+    __shared__ vec_t red[2][RED_SL][RED_OUT];
     __shared__ int nks[2][RED_MAXBLOCKS];
     const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
     int j = 0;
@@ -498,20 +514,25 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
             if (q < grp.n && (int)blockIdx.x >= grp.m[q].first_block) j = q;
     }
     const RedMat &r = grp.m[j];
-    // outputs are enumerated per token in runs of RED_OUT rows, so a workgroup never straddles tokens
+    // outputs are enumerated per token in runs of RUN rows, so a workgroup never straddles tokens
     const int local = blockIdx.x - r.first_block;
-    const int per_t = (r.M + RED_OUT - 1) / RED_OUT;
-    const int t = local / per_t, m0 = (local - t * per_t) * RED_OUT, m = m0 + lo;
-    const int rt = m0 / rows_per_tile;           // RED_OUT divides the tile height
-    const bool live = m < r.M;
+    const int per_t = (r.M + RUN - 1) / RUN;
+    const int t = local / per_t, m0 = (local - t * per_t) * RUN, m = m0 + VEC * lo;
+    const int rt = m0 / rows_per_tile;           // RUN divides the tile height
+    const bool live = m < r.M;                   // M % VEC == 0: all VEC outputs or none
     const bool two = grp.mode == EPI_SWIGLU;
     count_partials(r, rt, n_chunks, nks[0]);
     if (two) count_partials(grp.m[1], rt, n_chunks, nks[1]);
     // residual and bias do not depend on the sums: fetch them before the reduction
-    float extra = 0.f, res = 0.f;
+    float extra[VEC], res[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) { extra[e] = 0.f; res[e] = 0.f; }
     if (ks == 0 && live) {
-        if (r.bias) extra = (float)r.bias[m];
-        if (grp.mode == EPI_RESIDUAL) res = (float)residual[(int64_t)t * ldy + r.y_off + m];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            if (r.bias) extra[e] = (float)r.bias[m + e];
+            if (grp.mode == EPI_RESIDUAL) res[e] = (float)residual[(int64_t)t * ldy + r.y_off + m + e];
+        }
     }
     float scale = 1.f;
     __shared__ float ssq[RED_OUT * RED_SL / 64];
@@ -539,27 +560,31 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
         for (int w = 0; w < RED_OUT * RED_SL / 64; w++) q += ssq[w];
         scale = rsqrtf(q / (float)grp.n_in + grp.eps);
     }
-    red[0][ks][lo] = live ? slice_sum_any(r, T, t, m, ks, nks[0]) : 0.f;
-    if (two) red[1][ks][lo] = live ? slice_sum_any(grp.m[1], T, t, m, ks, nks[1]) : 0.f;
+    red[0][ks][lo] = live ? slice_sum_any<VEC>(r, T, t, m, ks, nks[0]) : vec_t(0.f);
+    if (two) red[1][ks][lo] = live ? slice_sum_any<VEC>(grp.m[1], T, t, m, ks, nks[1]) : vec_t(0.f);
     __syncthreads();
     if (ks != 0 || !live) return;
-    float s0 = 0.f;
+    vec_t s0 = vec_t(0.f), s1 = vec_t(0.f);
 #pragma unroll
     for (int k = 0; k < RED_SL; k++) s0 += red[0][k][lo];
-    s0 = s0 * scale + extra;
     if (two) {
-        float s1 = 0.f;
 #pragma unroll
         for (int k = 0; k < RED_SL; k++) s1 += red[1][k][lo];
-        s1 = s1 * scale + (grp.m[1].bias ? (float)grp.m[1].bias[m] : 0.f);
-        const float gate = (float)(half_t)s0, up = (float)(half_t)s1;
-        const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
-        y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
-        return;
     }
-    half_t v = (half_t)s0;
-    if (grp.mode == EPI_RESIDUAL) v = (half_t)(res + (float)v);
-    y[(int64_t)t * ldy + r.y_off + m] = v;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const float a0 = vec_get(s0, e) * scale + extra[e];
+        if (two) {
+            const float a1 = vec_get(s1, e) * scale + (grp.m[1].bias ? (float)grp.m[1].bias[m + e] : 0.f);
+            const float gate = (float)(half_t)a0, up = (float)(half_t)a1;
+            const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
+            y[(int64_t)t * ldy + m + e] = (half_t)((float)act * up);
+        } else {
+            half_t v = (half_t)a0;
+            if (grp.mode == EPI_RESIDUAL) v = (half_t)(res[e] + (float)v);
+            y[(int64_t)t * ldy + r.y_off + m + e] = v;
+        }
+    }
 }
 
 struct Plan {
@@ -713,15 +738,24 @@ int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T
     r.n_in = N;
     r.eps = eps;
     float *parts[GEMV_MAX_GROUP];
+    // many outputs (tokens x rows) and every M a multiple of 4: four outputs per thread
+    bool vec4 = true;
+    int64_t outputs = 0;
+    for (int j = 0; j < a.n; j++) {
+        vec4 = vec4 && a.M[j] % 4 == 0;
+        outputs += (int64_t)T * a.M[j];
+    }
+    vec4 = vec4 && outputs >= 32768;
+    const int run = vec4 ? 4 * RED_OUT : RED_OUT;
     int ldy = 0, blocks = 0;
     int64_t off = 0;
     for (int j = 0; j < a.n; j++) {
         const int groups = bs_strip_partials(a.I[j], a.M[j], N, K, T);
         parts[j] = part + off;
-        r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], (int)bs_cdiv(a.M[j], RED_OUT), 1, ldy, blocks, Split{1, 0}};
+        r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], (int)bs_cdiv(a.M[j], run), 1, ldy, blocks, Split{1, 0}};
         off += (int64_t)groups * T * a.M[j];
         ldy += a.M[j];
-        if (mode != EPI_SWIGLU || j == 0) blocks += T * (int)bs_cdiv(a.M[j], RED_OUT);
+        if (mode != EPI_SWIGLU || j == 0) blocks += T * (int)bs_cdiv(a.M[j], run);
     }
     r.ssq = input_rms ? part + off : nullptr;
     r.ssq_n = r.m[0].I;
@@ -730,7 +764,10 @@ int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T
     if (st != BS_OK) return st;
     if (mode == EPI_SWIGLU) ldy = a.M[0];
     for (int j = a.n; j < GEMV_MAX_GROUP; j++) r.m[j] = r.m[0];
-    gemv_reduce_kernel<<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, RED_OUT, 1);
+    if (vec4)
+        gemv_reduce_kernel<4><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, run, 1);
+    else
+        gemv_reduce_kernel<1><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, run, 1);
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
@@ -801,7 +838,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
                 if (mode != EPI_SWIGLU || j == 0) nblocks += tn * (int)bs_cdiv(a.M[j], RED_OUT);
             }
         }
-        gemv_reduce_kernel<<<nblocks, RED_OUT * RED_SL, 0, s>>>(rr, residual ? residual + (int64_t)t0 * ldy : nullptr,
+        gemv_reduce_kernel<1><<<nblocks, RED_OUT * RED_SL, 0, s>>>(rr, residual ? residual + (int64_t)t0 * ldy : nullptr,
                                                                 y + (int64_t)t0 * ldy, tn, ldy,
                                                                 p.waves * p.R * 16, p.n_chunks);
         BS_LAUNCH_CHECK();
