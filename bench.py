@@ -52,7 +52,7 @@ def parse():
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
     ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
-    ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..32)")
+    ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..48)")
     ap.add_argument("--prompt-len", type=int, default=2048, help="prompt tokens per sequence of --only decode_70b")
     ap.add_argument("--layer", default="14336x4096x16x1",
                     help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")

@@ -81,7 +81,7 @@ static int group_dims(const bs_matrix *mats, int n, int N, int K, int T) {
         if (st != BS_OK) return st;
         if (mats[j].I < 1) return BS_ERR_SHAPE;
     }
-    if (T < 1 || T > 32) return BS_ERR_SHAPE;
+    if (T < 1 || T > 48) return BS_ERR_SHAPE;
     return BS_OK;
 }
 

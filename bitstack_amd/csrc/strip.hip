@@ -221,7 +221,7 @@ struct StripPlan {
     size_t lds;
 };
 
-int token_tiles(int T) { return T <= 16 ? 1 : 2; }
+int token_tiles(int T) { return (T + 15) / 16; }
 
 size_t strip_lds(int I, int tt, int sg) {
     return ((size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
@@ -270,7 +270,7 @@ int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int 
 // Partial sums per output (groups of strips) when this path takes the shape, else 0.
 int bs_strip_partials(int I, int M, int N, int K, int T) {
     (void)K;
-    if (I < 1 || M < 1 || T < 1 || T > 32 || N % SF_COLS != 0) return 0;
+    if (I < 1 || M < 1 || T < 1 || T > 48 || N % SF_COLS != 0) return 0;
     if ((int64_t)M * N >= ((int64_t)1 << 34)) return 0;
     if (strip_lds(I, token_tiles(T), 1) > 160 * 1024) return 0;
     const StripPlan p = make_strip_plan(I, M, N, T);
@@ -297,5 +297,5 @@ int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *con
         if (p.lds > lds) lds = p.lds;
     }
     for (int j = n; j < STRIP_MAX_GROUP; j++) grp.m[j] = grp.m[0];
-    return token_tiles(T) == 1 ? launch_tt<1>(grp, slots, lds, x, N, K, T, s) : launch_tt<2>(grp, slots, lds, x, N, K, T, s);
+    return token_tiles(T) == 1 ? launch_tt<1>(grp, slots, lds, x, N, K, T, s) : token_tiles(T) == 2 ? launch_tt<2>(grp, slots, lds, x, N, K, T, s) : launch_tt<3>(grp, slots, lds, x, N, K, T, s);
 }

@@ -16,7 +16,7 @@ fused_level on this build:
   4  as 3 (deterministic; the reference's fp16 atomics are not reproduced)
      followed by the library's own MFMA linear instead of F.linear
   5  one C-ABI call for the whole forward: packed-sign MFMA GEMV for <= 4
-     tokens, weight patches rebuilt in registers for 5..32, rebuild-once +
+     tokens, weight patches rebuilt in registers for 5..48, rebuild-once +
      MFMA GEMM above.  Unlike the reference's level 5
      it takes any [..., N] input and a bias.
 Levels 1-5 need the tensors on a HIP device and the built shared library;

@@ -128,7 +128,7 @@ class MatrixGroup:
 
 
 def bitstack_forward_group_hip(group: MatrixGroup, x, epilogue=_lib.EPI_NONE, residual=None, out=None, rms_eps=None):
-    """All matrices of `group` applied to x [T, N] (T <= 32) in one launch, with
+    """All matrices of `group` applied to x [T, N] (T <= 48) in one launch, with
     the outputs side by side [T, sum M] (EPI_NONE), plus `residual` (EPI_RESIDUAL),
     or silu(first) * second [T, M] (EPI_SWIGLU).  What three (two) module calls and
     the element-wise ops after them do in a decoder layer.  With rms_eps set, x is

@@ -94,7 +94,7 @@ int64_t bs_workspace_bytes(int I, int M, int N, int K, int T);
  * (bitstack/utils/inference_utils.py:171-284).
  *
  * T <= 4 runs the packed-sign GEMV (signs contracted on MFMA against
- * vt_i o x, scaled by u_i, all blocks in one pass; N % 512 == 0); 5 <= T <= 32
+ * vt_i o x, scaled by u_i, all blocks in one pass; N % 512 == 0); 5 <= T <= 48
  * the strip kernel (16 x 16 patches of the weight rebuilt in registers and
  * multiplied by x at once, the weight never stored; N % 128 == 0; when it does
  * not take the shape, T <= 8 is two GEMV passes); larger T rebuilds the
@@ -131,7 +131,7 @@ int bs_linear_f16(const void *x, const void *w, const void *bias, void *y,
 
 /*
  * ---- decode step: several matrices per launch, fused epilogues -----------
- * One decode forward (T <= 32 tokens; more than 8 need N % 128 == 0) of up to 4 compressed matrices that read
+ * One decode forward (T <= 48 tokens; more than 8 need N % 128 == 0) of up to 4 compressed matrices that read
  * the same x, in one kernel pair: what q_proj/k_proj/v_proj (or gate_proj/
  * up_proj) of a decoder layer do with three (two) BitStackLinear.forward calls,
  * bitstack/modules/BitStackLinear.py:88-157, each as in bs_forward.  All share

@@ -47,7 +47,7 @@ def make_group(shapes, N, T, seed, bias=False):
 GROUP_CASES = [([(3, 512), (5, 128), (2, 128)], 512, 1), ([(3, 4096), (5, 1024), (2, 1024)], 4096, 1),
                ([(2, 1024), (4, 256)], 1024, 2), ([(1, 300), (2, 77), (3, 64), (1, 512)], 1536, 3),
                ([(2, 512), (3, 256)], 1024, 4), ([(2, 512), (1, 256)], 512, 5), ([(2, 256), (2, 256)], 1024, 8),
-               ([(2, 300), (3, 77), (1, 64)], 1536, 9), ([(3, 1024), (2, 256)], 4096, 16), ([(2, 200), (2, 200)], 384, 32)]
+               ([(2, 300), (3, 77), (1, 64)], 1536, 9), ([(3, 1024), (2, 256)], 4096, 16), ([(2, 200), (2, 200)], 384, 32), ([(2, 300), (1, 64)], 640, 48)]
 
 
 @pytest.mark.parametrize("shapes,N,T", GROUP_CASES)
@@ -94,7 +94,7 @@ def test_group_forward_swiglu(I0, I1, M, N, T):
 def test_group_rejects_what_the_decode_kernel_does_not_take():
     grp, x, _ = make_group([(1, 64), (1, 64)], 512, 1, seed=1)
     with pytest.raises(RuntimeError):
-        IU.bitstack_forward_group_hip(grp, torch.zeros(33, 512, dtype=torch.float16, device=dev()))   # more than 32 tokens
+        IU.bitstack_forward_group_hip(grp, torch.zeros(49, 512, dtype=torch.float16, device=dev()))   # more than 48 tokens
     grp2, _, _ = make_group([(1, 64), (1, 128)], 512, 1, seed=1)
     with pytest.raises(RuntimeError):
         IU.bitstack_forward_group_hip(grp2, x.to(dev()), _lib.EPI_SWIGLU)                               # unequal M

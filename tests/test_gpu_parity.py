@@ -164,10 +164,11 @@ def test_forward_odd_shapes_take_the_rebuild_path(I, M, N, T):
         assert_close(y, l0, "vs level-0 order")
 
 
-# 5..32 tokens: weight patches rebuilt in registers and multiplied at once (N a multiple of 128)
+# 5..48 tokens: weight patches rebuilt in registers and multiplied at once (N a multiple of 128)
 STRIP_CASES = [(1, 16, 128, 5, 16), (3, 100, 384, 9, 16), (2, 65, 1152, 17, 7), (4, 1000, 2048, 32, 16),
                (20, 64, 256, 6, 16), (2, 4096, 4096, 32, 16), (3, 14336, 4096, 8, 16), (2, 1024, 14336, 16, 16),
-               (36, 130, 128, 12, 3), (1, 4096, 1152, 8, 16), (2, 3000, 2432, 20, 16)]
+               (36, 130, 128, 12, 3), (1, 4096, 1152, 8, 16), (2, 3000, 2432, 20, 16),
+               (3, 1000, 1024, 33, 16), (2, 4096, 4096, 48, 16), (4, 333, 640, 41, 5)]
 
 
 @pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)

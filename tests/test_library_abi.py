@@ -83,8 +83,8 @@ def test_workspace_bytes(L):
     for T in (1, 4):
         b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
         assert b > 0 and b % (T * 4096 * 4) == 0 and b < 4096 * 4096 * 2
-    # 5..32 tokens: partial sums per group of strips (plus the groups' sums of squares of x)
-    for T in (8, 32):
+    # 5..48 tokens: partial sums per group of strips (plus the groups' sums of squares of x)
+    for T in (8, 32, 48):
         b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
         assert T * 4096 * 4 <= b <= 32 * (T * 4096 * 4 + T * 4) + 256
 
@@ -98,8 +98,8 @@ def test_group_and_decode_step_validation(L):
     assert L.bs_forward_group_workspace_bytes(mats, 2, 500, 16, 1) == -2          # N % 8
     assert L.bs_forward_group_workspace_bytes(mats, 2, 520, 16, 1) == -2          # not a decode-kernel shape
     assert L.bs_forward_group_workspace_bytes(mats, 5, 512, 16, 1) == -2          # more than BS_MAX_GROUP
-    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 9) > 0            # 9..32 tokens: the strip kernel
-    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 33) == -2         # more than 32 tokens
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 9) > 0            # 9..48 tokens: the strip kernel
+    assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 16, 49) == -2         # more than 48 tokens
     assert L.bs_forward_group_workspace_bytes(mats, 2, 512, 17, 1) == -3
     assert L.bs_forward_group_workspace_bytes(nul, 2, 512, 16, 1) == -1
     big = 1 << 30
