@@ -391,13 +391,17 @@ int bs_launch_attention_decode(const half_t *qkv, half_t *kcache, half_t *vcache
                                const int64_t *pos, half_t *out, int B, int heads, int kv_heads, int head_dim,
                                int max_len, hipStream_t s) {
     if (head_dim != ATT_D || max_len > ATT_MAX_LEN) return BS_ERR_SHAPE;
-    // Long caches: four (or two) query heads of a KV head per workgroup, a quarter (half) of
-    // the cache fetches; short ones are latency bound and do better with a workgroup per head.
+    // Long caches and more (head, sequence) pairs than CUs: four (or two) query heads of a KV
+    // head per workgroup, a quarter (half) of the cache fetches.  A workgroup of the grouped
+    // kernel takes longer than one of the per-head kernel (3000 positions: 55 us against 25),
+    // so it only pays once the per-head kernel would need more than one round of workgroups
+    // (8 sequences x 64 heads at 2100 positions: 45 us against 79).
     const int rep = heads / kv_heads;
-    if (max_len >= 1024 && rep % 4 == 0)
+    const bool grouped = max_len >= 1024 && (int64_t)B * heads > 256;
+    if (grouped && rep % 4 == 0)
         attention_decode_gqa_kernel<4><<<dim3(heads / 4, B), GQA_THREADS, 0, s>>>(qkv, kcache, vcache, cos, sin, pos, out,
                                                                                  heads, kv_heads, max_len);
-    else if (max_len >= 1024 && rep % 2 == 0)
+    else if (grouped && rep % 2 == 0)
         attention_decode_gqa_kernel<2><<<dim3(heads / 2, B), GQA_THREADS, 0, s>>>(qkv, kcache, vcache, cos, sin, pos, out,
                                                                                  heads, kv_heads, max_len);
     else

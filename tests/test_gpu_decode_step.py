@@ -117,8 +117,9 @@ def test_rmsnorm(T, H):
 
 
 @pytest.mark.parametrize("B,heads,kv,max_len", [(1, 32, 8, 40), (3, 4, 2, 40), (2, 8, 8, 40), (2, 16, 2, 40), (1, 6, 2, 40),
-                                                # long caches: several query heads of a KV head per workgroup
-                                                (2, 16, 2, 1100), (1, 32, 8, 1024), (2, 4, 2, 2048), (1, 6, 2, 1500)])
+                                                # long caches; with more than 256 (head, sequence) pairs several
+                                                # query heads of a KV head share a workgroup
+                                                (2, 16, 2, 1100), (1, 32, 8, 1024), (9, 32, 8, 1100), (17, 16, 8, 1024), (33, 8, 8, 1024)])
 def test_attention_decode_steps(B, heads, kv, max_len):
     print(f"attention B={B} heads={heads} kv={kv} max_len={max_len}", flush=True)
     d, steps = 128, 37
@@ -150,7 +151,7 @@ def test_attention_decode_steps(B, heads, kv, max_len):
 
 
 @pytest.mark.parametrize("B,heads,kv,max_len,at", [(2, 16, 2, 2048, 1500), (1, 8, 4, 1024, 1023), (1, 32, 8, 4096, 3000),
-                                                   (1, 4, 1, 1200, 517)])
+                                                   (5, 64, 8, 2048, 1500), (9, 32, 16, 1024, 1023), (3, 96, 8, 1200, 517)])
 def test_attention_decode_deep_in_a_long_cache(B, heads, kv, max_len, at):
     """One step at position `at` of a cache already holding random rows."""
     print(f"attention deep B={B} heads={heads} kv={kv} max_len={max_len} at={at}", flush=True)
@@ -187,10 +188,11 @@ def test_attention_position_outside_the_cache_writes_zeros_and_touches_nothing()
     qkv = torch.ones(1, 8 * 128, dtype=torch.float16, device=dev())
     out = IU.attention_decode_hip(qkv, kc, vc, tab, tab, torch.tensor([8], device=dev()), 4, 2)
     assert float(out.abs().max()) == 0.0 and float(kc.abs().max()) == 0.0
-    # the same through the grouped-query kernel of long caches
-    kc = torch.zeros(1, 2, 1024, 128, dtype=torch.float16, device=dev())
+    # the same through the grouped-query kernel (long cache, more than 256 (head, sequence) pairs)
+    kc = torch.zeros(65, 2, 1024, 128, dtype=torch.float16, device=dev())
     vc = torch.zeros_like(kc)
     tab = torch.ones(1024, 64, dtype=torch.float16, device=dev())
+    qkv = torch.ones(65, 8 * 128, dtype=torch.float16, device=dev())
     out = IU.attention_decode_hip(qkv, kc, vc, tab, tab, torch.tensor([1024], device=dev()), 4, 2)
     assert float(out.abs().max()) == 0.0 and float(kc.abs().max()) == 0.0
 
