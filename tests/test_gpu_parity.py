@@ -261,6 +261,31 @@ def build_module(M, N, I, bias, seed):
     return mod, x
 
 
+def test_full_size_properties_strip_kernel():
+    """The same for the 5..48-token path at 14336 x 4096 with 8 blocks."""
+    I, M, N = 8, 14336, 4096
+    q, u, vt, x = synthetic_layer(M, N, I, 16, seed=10, device=dev())
+    f = IU.bitstack_forward_hip
+    assert _lib.decode_plan(I, M, N, 16, 16)[0] == 0
+    y = f(q, u, vt, x)
+    assert torch.equal(f(q, u, vt, x), y)                                   # determinism
+    # tokens do not interact: the first eight rows are the 8-token answer, bit for bit
+    assert torch.equal(f(q, u, vt, x[:8].contiguous()), y[:8])
+    # and a 40-token call (three token tiles) repeats them
+    x40 = torch.cat([x, x, x[:8]])
+    y40 = f(q, u, vt, x40)
+    assert torch.equal(y40[:16], y) and torch.equal(y40[16:32], y) and torch.equal(y40[32:], y[:8])
+    yf = y.float()
+    scale = float(yf.abs().max())
+    assert float((f(q, u, vt, x * 2).float() - 2 * yf).abs().max()) <= 2e-3 * scale           # linearity in x
+    parts = f(q[:4], u[:4], vt[:4], x).float() + f(q[4:], u[4:], vt[4:], x).float()
+    assert float((parts - yf).abs().max()) <= 4e-3 * scale                                    # block additivity (w is rounded per call)
+    assert float((f(~q, u, vt, x).float() + yf).abs().max()) <= 1e-3 * scale                  # complemented signs negate
+    # the decode kernel gives the same numbers up to the rounding points (it never rounds w)
+    y1 = torch.cat([f(q, u, vt, x[t:t + 1].contiguous()) for t in range(4)]).float()
+    assert float((y1 - yf[:4]).abs().max()) <= 4e-3 * scale
+
+
 @pytest.mark.parametrize("bias", [False, True])
 def test_module_levels_agree_with_level0(bias):
     M, N, I = 256, 1024, 4
