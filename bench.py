@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
-    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer"], default=None,
+    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer", "scoring"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..48)")
     ap.add_argument("--prompt-len", type=int, default=2048, help="prompt tokens per sequence of --only decode_70b")
@@ -149,6 +149,28 @@ def e2e_decode_70b(torch, dev, batch=8, prompt_len=2048, new_tokens=128):
             "hbm_roofline_tok_s": round(batch * 8e12 / wbytes, 1),
             "config": f"80 layers, hidden 8192, inter 28672, 64Q/8KV, vocab 128256, batch {batch}, {prompt_len}-token prompt in one "
                       f"pass, {new_tokens} greedy tokens per sequence, fused step, one HIP-graph replay per step"}
+
+
+def scoring_eval(torch, dev, sequences=8, seqlen=2048, blocks=4):
+    """One perplexity evaluation of the importance-scoring loop on the 8B shape: every linear
+    with `blocks` blocks, `sequences` calibration sequences of `seqlen` random token ids through
+    the one-pass forward (rebuild + dense kernels) and a cross entropy over all positions.  The
+    loop itself is one such evaluation per (bit level, linear)."""
+    from bitstack_amd.utils.llama_decode import LLAMA_8B, PROJ, SyntheticLlamaDecoder
+    from bitstack_amd.utils import scoring
+    cfg = {f"layer.{L}.{p}": blocks for L in range(LLAMA_8B.layers) for p in PROJ}
+    model = SyntheticLlamaDecoder(LLAMA_8B, cfg, seqlen, dev, batch=4)
+    ids = torch.randint(0, LLAMA_8B.vocab, (sequences, seqlen), generator=torch.Generator().manual_seed(0))
+    scoring.eval_ppl(model, ids[:4])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ppl = scoring.eval_ppl(model, ids)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    n_lin = LLAMA_8B.layers * len(PROJ)
+    return {"seconds_per_evaluation": round(dt, 3), "tokens_per_s": round(sequences * seqlen / dt, 1), "ppl_random_init": round(ppl, 1),
+            "evaluations_per_bit_level": n_lin, "minutes_per_bit_level": round(n_lin * dt / 60, 1),
+            "config": f"8B shape, {blocks} blocks per linear, {sequences} sequences x {seqlen} tokens, batch 4"}
 
 
 def e2e_decode(torch, dev, prompt_len=128, new_tokens=256):
@@ -315,6 +337,9 @@ def main():
         return
     if a.only == "decode_8b":
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
+        return
+    if a.only == "scoring":
+        print(json.dumps({"scoring": scoring_eval(torch, dev)}))
         return
     if a.only == "decode_70b":
         print(json.dumps({"decode_70b": e2e_decode_70b(torch, dev, batch=a.batch, prompt_len=a.prompt_len)}))

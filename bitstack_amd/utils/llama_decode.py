@@ -301,11 +301,12 @@ class SyntheticLlamaDecoder:
         self.pos.add_(1)
 
     @torch.no_grad()
-    def prefill(self, prompt: torch.Tensor):
+    def prefill(self, prompt: torch.Tensor, all_logits=False):
         """The whole prompt [batch, len] in one pass: every linear sees batch * len tokens (the
         library's rebuild + dense path), causal attention and RoPE are torch ops, the KV cache
         is filled for positions 0 .. len - 1, and self.token becomes the greedy token after
-        the prompt.  Decode continues from there with step() or step_fused()."""
+        the prompt.  Decode continues from there with step() or step_fused().  With
+        all_logits the logits of every position [batch, len, vocab] are returned (perplexity)."""
         s, B = self.s, self.batch
         prompt = prompt.view(1, -1).expand(B, -1) if prompt.dim() == 1 else prompt
         n = prompt.shape[1]
@@ -332,10 +333,15 @@ class SyntheticLlamaDecoder:
             act = F.silu(lin["mlp.gate_proj"](hn))
             act.mul_(lin["mlp.up_proj"](hn))
             x = x + lin["mlp.down_proj"](act)
-        last = x.view(B, n, s.hidden)[:, -1].contiguous()
-        self.logits = F.linear(rmsnorm_hip(last, self.final_norm, s.rms_eps), self.lm_head)
+        if all_logits:
+            full = F.linear(rmsnorm_hip(x, self.final_norm, s.rms_eps), self.lm_head).view(B, n, -1)
+            self.logits = full[:, -1].contiguous()
+        else:
+            last = x.view(B, n, s.hidden)[:, -1].contiguous()
+            self.logits = F.linear(rmsnorm_hip(last, self.final_norm, s.rms_eps), self.lm_head)
         self.token.copy_(self.logits.argmax(-1))
         self.pos.fill_(n)
+        return full if all_logits else None
 
     def prefill_positions(self, prompt: torch.Tensor, fused=False):
         """Feed a prompt token by token (the measurement is about decode).  `prompt`

@@ -381,3 +381,55 @@ def test_argmax(B, V):
     got = IU.argmax_hip(x.to(dev())).cpu()
     row = x[0].float().numpy().copy(); row[3] = -np.inf
     assert int(got[0]) == int(np.argmax(row))       # NaN never wins
+
+
+def test_importance_scoring_and_compression_configs(tmp_path):
+    """The scoring loop on a small decoder: perplexity against the float64 decoder, one entry per
+    (bit level, linear), block counts restored, and configs whose memory grows by the scored
+    linear's bytes per block and which the checkpoint reader accepts."""
+    from bitstack_amd.utils import checkpoint as ck
+    from bitstack_amd.utils import scoring as S
+    niter = 3
+    cfg = {f"layer.{L}.{p}": niter for L in range(SMALL.layers) for p in PROJ}
+    m = SyntheticLlamaDecoder(SMALL, cfg, 32, dev(), seed=8, batch=2)
+    with torch.no_grad():
+        m.embed.mul_(30.0)
+    ids = torch.randint(0, SMALL.vocab, (3, 12), generator=torch.Generator().manual_seed(5))
+    # perplexity of the full model against the float64 decoder
+    w = dense_weights(m)
+    nll = []
+    for s_ in range(ids.shape[0]):
+        orc = LO.LlamaOracle(w, SMALL.layers, SMALL.heads, SMALL.kv_heads, SMALL.head_dim, SMALL.rope_theta, SMALL.rms_eps, 32)
+        tot = 0.0
+        for j in range(ids.shape[1] - 1):
+            lg = orc.step(int(ids[s_, j]))
+            lg = lg - lg.max()
+            tot += -(lg[int(ids[s_, j + 1])] - np.log(np.exp(lg).sum()))
+        nll.append(tot / (ids.shape[1] - 1))
+    want = float(np.exp(np.mean(nll)))
+    got = S.eval_ppl(m, ids)
+    assert abs(got - want) <= 2e-2 * want, (got, want)
+
+    seen = []
+    scores = S.score_importance(m, ids, niter, progress=lambda bit, name, ppl: seen.append((bit, name)))
+    names = [n for n, _ in S.all_linears(m)]
+    assert len(names) == SMALL.layers * len(PROJ)
+    assert abs(scores["original_ppl"] - got) <= 1e-6 * got
+    assert [lvl["bit"] for lvl in scores["reduced_ppl"]] == [1, 2]
+    for lvl in scores["reduced_ppl"]:
+        assert [e["layer"] for e in lvl["ppls"]] == names and all(np.isfinite(e["ppl"]) for e in lvl["ppls"])
+    assert len(seen) == 2 * len(names)
+    assert all(mod.w_bit == niter for _, mod in S.all_linears(m))          # restored
+    configs = S.compression_configs_for(m, scores)
+    assert len(configs) == 1 + 2 * len(names)
+    per_bit = {n: int(mod.memory_per_bit()) for n, mod in S.all_linears(m)}
+    order = S.sort_layers_and_bits_average(scores)
+    for a, b, name in zip(configs[:-1], configs[1:], order):
+        assert b["memory"] - a["memory"] == per_bit[name]
+        assert b["layers"][name] == a["layers"][name] + 1
+    assert configs[-1]["layers"] == {n: niter for n in names}
+    assert configs[-1]["memory"] == m.weight_bytes() + (m.norm_w.numel() + m.final_norm.numel()) * 2
+    S.save_scores_and_configs(str(tmp_path), scores, configs)
+    again = ck.read_compression_configs(str(tmp_path))
+    mid = configs[len(configs) // 2]
+    assert ck.retrieve_compression_config(again, mid["memory"] / 1024 ** 2 + 1e-6) == mid["layers"]

@@ -147,3 +147,35 @@ def test_unpack_sign_v2_is_the_same_mapping_with_a_dtype_check():
         assert np.array_equal(got, want)
     with pytest.raises(ValueError):
         unpack_sign_v2(packed.to(torch.int16), torch.Size((8,)))
+
+
+# ------------------------------------------------------------------ importance scores -> configs
+def test_sort_layers_and_generate_configs():
+    """Hand-checked: within a bit level the linear with the lowest perplexity comes first,
+    levels follow one another, a NaN borrows the next level's value plus the level's maximum
+    (model_utils.py:26-66)."""
+    from bitstack_amd.utils import scoring as S
+    data = {"original_ppl": 9.0, "reduced_ppl": [
+        {"bit": 1, "ppls": [{"layer": "a", "ppl": 7.0}, {"layer": "b", "ppl": 5.0}, {"layer": "c", "ppl": 6.0}]},
+        {"bit": 2, "ppls": [{"layer": "a", "ppl": 4.0}, {"layer": "b", "ppl": 4.5}, {"layer": "c", "ppl": 3.0}]}]}
+    assert S.sort_layers_and_bits_average(data) == ["b", "c", "a", "c", "a", "b"]
+    per_bit = {"a": 10, "b": 20, "c": 30}
+    cfgs = S.generate_configs(["b", "c", "a", "c", "a", "b"], per_bit, 100)
+    assert [c["memory"] for c in cfgs] == [100, 120, 150, 160, 190, 200, 220]
+    assert cfgs[0]["layers"] == {"a": 1, "b": 1, "c": 1} and cfgs[-1]["layers"] == {"a": 3, "b": 3, "c": 3}
+    assert cfgs[2]["layers"] == {"a": 1, "b": 2, "c": 2}
+    # a NaN at level 1 sorts by the next level's perplexity, after every finite entry
+    nan = {"reduced_ppl": [
+        {"bit": 1, "ppls": [{"layer": "a", "ppl": float("nan")}, {"layer": "b", "ppl": 5.0}, {"layer": "c", "ppl": float("nan")}]},
+        {"bit": 2, "ppls": [{"layer": "a", "ppl": 4.0}, {"layer": "b", "ppl": 4.5}, {"layer": "c", "ppl": 3.0}]}]}
+    assert S.sort_layers_and_bits_average(nan)[:3] == ["c", "a", "b"]      # 3.0 + 0, 4.0 + 0, 5.0 (the reference's NaN-poisoned max is 0)
+    nan2 = {"reduced_ppl": [
+        {"bit": 1, "ppls": [{"layer": "a", "ppl": 6.0}, {"layer": "b", "ppl": float("nan")}, {"layer": "c", "ppl": 5.0}]},
+        {"bit": 2, "ppls": [{"layer": "a", "ppl": 4.0}, {"layer": "b", "ppl": 0.5}, {"layer": "c", "ppl": 3.0}]}]}
+    assert S.sort_layers_and_bits_average(nan2)[:3] == ["c", "a", "b"]     # b: 0.5 + 6.0 sorts after the finite ones
+    bad = {"reduced_ppl": [{"bit": 1, "ppls": [{"layer": "a", "ppl": float("nan")}]}]}
+    with pytest.raises(ValueError):
+        S.sort_layers_and_bits_average(bad)
+    # the list is what retrieve_compression_config reads
+    from bitstack_amd.utils import checkpoint as ck
+    assert ck.retrieve_compression_config(cfgs, 155 / 1024 ** 2) == cfgs[2]["layers"]
