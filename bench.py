@@ -167,9 +167,27 @@ def scoring_eval(torch, dev, sequences=8, seqlen=2048, blocks=4):
     ppl = scoring.eval_ppl(model, ids)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    # the loop resumes every evaluation at its linear's layer: time it for the first, the middle
+    # and the last decoder layer (inputs of all layers kept from one full run per batch)
+    batches = scoring._batches(model, ids)
+    kept = []
+    for b_ids, _ in batches:
+        keep = []
+        model.prefill(b_ids, keep=keep)
+        kept.append(keep)
+    resumed = {}
+    for L in (0, LLAMA_8B.layers // 2, LLAMA_8B.layers - 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for b, (b_ids, real) in enumerate(batches):
+            scoring._nll(model.prefill(b_ids, all_logits=True, first_layer=L, hidden=kept[b][L] if L else None), b_ids, real)
+        torch.cuda.synchronize()
+        resumed[f"from_layer_{L}"] = round(time.perf_counter() - t0, 3)
+    mean_resumed = sum(resumed.values()) / len(resumed)
     n_lin = LLAMA_8B.layers * len(PROJ)
     return {"seconds_per_evaluation": round(dt, 3), "tokens_per_s": round(sequences * seqlen / dt, 1), "ppl_random_init": round(ppl, 1),
-            "evaluations_per_bit_level": n_lin, "minutes_per_bit_level": round(n_lin * dt / 60, 1),
+            "seconds_per_resumed_evaluation": resumed,
+            "evaluations_per_bit_level": n_lin, "minutes_per_bit_level": round(n_lin * mean_resumed / 60, 1),
             "config": f"8B shape, {blocks} blocks per linear, {sequences} sequences x {seqlen} tokens, batch 4"}
 
 

@@ -301,21 +301,31 @@ class SyntheticLlamaDecoder:
         self.pos.add_(1)
 
     @torch.no_grad()
-    def prefill(self, prompt: torch.Tensor, all_logits=False):
+    def prefill(self, prompt: torch.Tensor, all_logits=False, first_layer=0, hidden=None, keep=None):
         """The whole prompt [batch, len] in one pass: every linear sees batch * len tokens (the
         library's rebuild + dense path), causal attention and RoPE are torch ops, the KV cache
         is filled for positions 0 .. len - 1, and self.token becomes the greedy token after
         the prompt.  Decode continues from there with step() or step_fused().  With
-        all_logits the logits of every position [batch, len, vocab] are returned (perplexity)."""
+        all_logits the logits of every position [batch, len, vocab] are returned (perplexity).
+        `keep` (a list) receives the input of every decoder layer; `first_layer` with `hidden`
+        (such a kept input) resumes from that layer - what a change confined to one layer needs
+        to be evaluated (the KV cache of the earlier layers is then left as it is)."""
         s, B = self.s, self.batch
         prompt = prompt.view(1, -1).expand(B, -1) if prompt.dim() == 1 else prompt
         n = prompt.shape[1]
         if n < 1 or n > self.max_len:
             raise ValueError("prompt length must be in 1..max_len")
         d = s.head_dim
-        x = self.embed.index_select(0, prompt.reshape(-1))                # [B * n, h]
+        if first_layer == 0:
+            x = self.embed.index_select(0, prompt.reshape(-1))            # [B * n, h]
+        else:
+            if hidden is None or tuple(hidden.shape) != (B * n, s.hidden):
+                raise ValueError("resuming needs the kept input of that layer")
+            x = hidden
         cos, sin = self.cos[:n].view(1, 1, n, d // 2), self.sin[:n].view(1, 1, n, d // 2)
-        for L in range(s.layers):
+        for L in range(first_layer, s.layers):
+            if keep is not None:
+                keep.append(x)
             lin = self.lin[L]
             hn = rmsnorm_hip(x, self.norm_w[L, 0], s.rms_eps)
             q = lin["self_attn.q_proj"](hn).view(B, n, s.heads, d).transpose(1, 2)

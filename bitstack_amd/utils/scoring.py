@@ -18,21 +18,35 @@ import torch
 import torch.nn.functional as F
 
 
-@torch.no_grad()
-def eval_ppl(decoder, input_ids: torch.Tensor) -> float:
-    """exp(mean over sequences of the mean next-token negative log-likelihood), as
-    model_utils.py:117-133.  `input_ids` is [n_sequences, seqlen]; sequences are run in
-    batches of the decoder's batch size (the last batch is padded by repeating rows)."""
+def _batches(decoder, input_ids):
+    """[(ids [B, n] on the device, number of real rows)]: the last batch is padded by repeating rows."""
     B = decoder.batch
-    nlls = []
+    out = []
     for i in range(0, input_ids.shape[0], B):
         ids = input_ids[i:i + B].to(decoder.dev)
         real = ids.shape[0]
         if real < B:
             ids = torch.cat([ids, ids[-1:].expand(B - real, -1)])
-        logits = decoder.prefill(ids, all_logits=True)                    # [B, n, vocab]
-        loss = F.cross_entropy(logits[:, :-1].float().permute(0, 2, 1), ids[:, 1:], reduction="none")
-        nlls.append(loss.mean(dim=1)[:real])
+        out.append((ids, real))
+    return out
+
+
+def _nll(logits, ids, real):
+    """Mean next-token negative log-likelihood per sequence (fp32 log-softmax, one sequence at a
+    time so that the fp32 copy of the logits stays small)."""
+    out = []
+    for b in range(real):
+        loss = F.cross_entropy(logits[b, :-1].float(), ids[b, 1:], reduction="none")
+        out.append(loss.mean())
+    return torch.stack(out)
+
+
+@torch.no_grad()
+def eval_ppl(decoder, input_ids: torch.Tensor) -> float:
+    """exp(mean over sequences of the mean next-token negative log-likelihood), as
+    model_utils.py:117-133.  `input_ids` is [n_sequences, seqlen]; sequences are run in
+    batches of the decoder's batch size."""
+    nlls = [_nll(decoder.prefill(ids, all_logits=True), ids, real) for ids, real in _batches(decoder, input_ids)]
     return float(torch.exp(torch.cat(nlls).mean()))
 
 
@@ -45,31 +59,57 @@ def all_linears(decoder):
     return out
 
 
+def all_linears_with_layer(decoder):
+    out = []
+    for L, row in enumerate(decoder.lin):
+        for p, m in row.items():
+            out.append((getattr(m, "name", None) or f"layer.{L}.{p}", m, L))
+    return out
+
+
 @torch.no_grad()
-def score_importance(decoder, input_ids: torch.Tensor, niter: int, progress=None):
+def score_importance(decoder, input_ids: torch.Tensor, niter: int, progress=None, reuse_prefix=True):
     """For bit = 1 .. niter - 1: every linear at `bit` blocks, then one linear at a time at
     bit + 1 and the calibration perplexity with it (main.py:146-157).  Returns the dict the
-    reference writes to reduced_ppl_average.json.  The block counts are restored."""
-    linears = all_linears(decoder)
-    saved = [m.w_bit for _, m in linears]
+    reference writes to reduced_ppl_average.json.  The block counts are restored.
+
+    reuse_prefix: a linear of decoder layer L changes nothing before layer L, so per bit
+    level the input of every layer is kept from one run at the level's block counts and each
+    evaluation resumes at its linear's layer - the same numbers for about half the work
+    (batches x layers x batch x seqlen x hidden fp16 values are held meanwhile)."""
+    linears = all_linears_with_layer(decoder)
+    saved = [m.w_bit for _, m, _ in linears]
+    batches = _batches(decoder, input_ids)
     try:
         original = eval_ppl(decoder, input_ids)
         ppls = []
         for bit in range(1, niter):
-            for _, m in linears:
+            for _, m, _ in linears:
                 m.set_bit(bit)
+            kept = []
+            if reuse_prefix:
+                for ids, _ in batches:
+                    keep = []
+                    decoder.prefill(ids, keep=keep)
+                    kept.append(keep)
             per_bit = []
-            for name, m in linears:
+            for name, m, L in linears:
                 m.set_bit(bit + 1)
-                ppl = eval_ppl(decoder, input_ids)
+                if reuse_prefix:
+                    nlls = [_nll(decoder.prefill(ids, all_logits=True, first_layer=L, hidden=kept[b][L] if L else None), ids, real)
+                            for b, (ids, real) in enumerate(batches)]
+                    ppl = float(torch.exp(torch.cat(nlls).mean()))
+                else:
+                    ppl = eval_ppl(decoder, input_ids)
                 m.set_bit(bit)
                 per_bit.append({"layer": name, "ppl": ppl})
                 if progress is not None:
                     progress(bit, name, ppl)
             ppls.append({"bit": bit, "ppls": per_bit})
+            del kept
         return {"original_ppl": original, "reduced_ppl": ppls}
     finally:
-        for (_, m), b in zip(linears, saved):
+        for (_, m, _), b in zip(linears, saved):
             m.set_bit(b)
 
 

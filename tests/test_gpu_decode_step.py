@@ -412,6 +412,9 @@ def test_importance_scoring_and_compression_configs(tmp_path):
 
     seen = []
     scores = S.score_importance(m, ids, niter, progress=lambda bit, name, ppl: seen.append((bit, name)))
+    # resuming every evaluation at its linear's layer gives the very same numbers
+    plain = S.score_importance(m, ids, niter, reuse_prefix=False)
+    assert plain == scores
     names = [n for n, _ in S.all_linears(m)]
     assert len(names) == SMALL.layers * len(PROJ)
     assert abs(scores["original_ppl"] - got) <= 1e-6 * got
