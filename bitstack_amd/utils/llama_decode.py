@@ -178,6 +178,43 @@ class SyntheticLlamaDecoder:
         self._setup(shape, lin, embed, lm_head, norm_w, f16(other["model.norm.weight"]), max_len, dev, batch)
         return self
 
+    @classmethod
+    def from_dense(cls, shape: LlamaShape, weights: dict, niter: int, max_len: int, device, k=16, batch=1):
+        """Compress a dense Llama: every decoder linear becomes a BitStackLinear with `niter`
+        residual blocks of rank `k`, decomposed on the device one linear at a time (what
+        bitstack/utils/decompose.py:8-31 does to the Hugging Face model with
+        BitStackLinear.from_linear; names layer.{L}.{proj} as there).  `weights` uses the
+        Hugging Face keys: model.layers.{L}.{proj}.weight, the two layer norms per layer,
+        model.embed_tokens.weight, model.norm.weight and lm_head.weight (optional: tied)."""
+        import dataclasses
+        dev = torch.device(device)
+        shape = dataclasses.replace(shape, k=k)
+        f16 = lambda t: torch.as_tensor(t).to(dev, torch.float16).contiguous()
+        lin = []
+        for L in range(shape.layers):
+            row = {}
+            for p in PROJ:
+                w = torch.as_tensor(weights[f"model.layers.{L}.{p}.weight"]).to(dev, torch.float32)
+                m, n = shape.proj_shape(p)
+                if tuple(w.shape) != (m, n):
+                    raise ValueError(f"model.layers.{L}.{p}.weight is {tuple(w.shape)}, expected {(m, n)}")
+                dense = torch.nn.Linear(n, m, bias=False, device=dev, dtype=torch.float16)
+                with torch.no_grad():
+                    dense.weight.copy_(w)
+                    mod = BitStackLinear.from_linear(dense, w_bit=niter, k=k, bias=False, fused_level=5, name=f"layer.{L}.{p}")
+                mod.stack_blocks()
+                row[p] = mod
+                del dense, w
+            lin.append(row)
+        norm_w = torch.stack([torch.stack([f16(weights[f"model.layers.{L}.input_layernorm.weight"]),
+                                           f16(weights[f"model.layers.{L}.post_attention_layernorm.weight"])])
+                              for L in range(shape.layers)])
+        embed = f16(weights["model.embed_tokens.weight"])
+        lm_head = f16(weights["lm_head.weight"]) if "lm_head.weight" in weights else embed
+        self = cls.__new__(cls)
+        self._setup(shape, lin, embed, lm_head, norm_w, f16(weights["model.norm.weight"]), max_len, dev, batch)
+        return self
+
     def save_checkpoint(self, path, compression_configs=None, max_shard_bytes=None):
         """Writes this decoder in the same layout (config.json included)."""
         import json
@@ -202,6 +239,17 @@ class SyntheticLlamaDecoder:
             for m in row.values():
                 b += m.qweight.numel() + 2 * (m.u.numel() + m.vt.numel())
         return b
+
+    def set_bits(self, bits):
+        """Blocks in use per linear from now on: one count for all, or {"layer.{L}.{proj}": count}
+        (BitStackLinear.set_bit on each; the grouped launches' argument blocks are rebuilt)."""
+        for L, row in enumerate(self.lin):
+            for p, m in row.items():
+                b = bits if isinstance(bits, int) else bits[f"layer.{L}.{p}"]
+                if not 1 <= b <= m.u.shape[0]:
+                    raise ValueError(f"layer.{L}.{p}: {b} blocks asked, {m.u.shape[0]} loaded")
+                m.set_bit(b)
+        self._groups = None
 
     def reset(self):
         self.pos.zero_()

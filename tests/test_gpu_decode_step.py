@@ -436,3 +436,74 @@ def test_importance_scoring_and_compression_configs(tmp_path):
     again = ck.read_compression_configs(str(tmp_path))
     mid = configs[len(configs) // 2]
     assert ck.retrieve_compression_config(again, mid["memory"] / 1024 ** 2 + 1e-6) == mid["layers"]
+
+
+def test_whole_flow_dense_to_compressed_to_budgeted_decoder(tmp_path):
+    """Dense random Llama -> from_dense (decompose on the device) -> decode against the float64
+    decoder on the DENSE weights, closer with every block kept -> checkpoint round trip ->
+    importance scores -> compression configs -> a decoder loaded at a memory budget."""
+    from bitstack_amd.utils import checkpoint as ck
+    from bitstack_amd.utils import scoring as S
+    print("whole flow: dense -> compressed -> scored -> budgeted", flush=True)
+    niter = 4
+    g = torch.Generator().manual_seed(21)
+    w = {"model.embed_tokens.weight": torch.randn(SMALL.vocab, SMALL.hidden, generator=g),
+         "lm_head.weight": torch.randn(SMALL.vocab, SMALL.hidden, generator=g) * SMALL.hidden ** -0.5,
+         "model.norm.weight": 1 + 0.1 * torch.randn(SMALL.hidden, generator=g)}
+    for L in range(SMALL.layers):
+        w[f"model.layers.{L}.input_layernorm.weight"] = 1 + 0.1 * torch.randn(SMALL.hidden, generator=g)
+        w[f"model.layers.{L}.post_attention_layernorm.weight"] = 1 + 0.1 * torch.randn(SMALL.hidden, generator=g)
+        for p in PROJ:
+            m_, n_ = SMALL.proj_shape(p)
+            w[f"model.layers.{L}.{p}.weight"] = torch.randn(m_, n_, generator=g) * n_ ** -0.5
+    w = {k_: v.half().float() for k_, v in w.items()}          # what a fp16 checkpoint would hold
+    model = SyntheticLlamaDecoder.from_dense(SMALL, w, niter, 16, dev())
+    assert all(m.w_bit == niter and m.u.shape[0] == niter and m.name == f"layer.{L}.{p}"
+               for L, row in enumerate(model.lin) for p, m in row.items())
+    # every block kept brings each rebuilt weight closer to the dense one (float64 rebuild)
+    for L in (0, 1):
+        for p in ("self_attn.k_proj", "mlp.down_proj"):
+            m = model.lin[L][p]
+            dense = w[f"model.layers.{L}.{p}.weight"].double().numpy()
+            errs = [np.linalg.norm(O.reconstruct_w_exact(m.qweight[:b].cpu().numpy(), m.u[:b].cpu().numpy(), m.vt[:b].cpu().numpy()) - dense)
+                    / np.linalg.norm(dense) for b in range(1, niter + 1)]
+            assert all(errs[i + 1] < 0.8 * errs[i] for i in range(niter - 1)) and errs[-1] < 0.2, errs
+    # decode against the float64 decoder on the dense weights: the gap shrinks with the blocks
+    toks = [7, 130, 22, 201, 64]
+    orc = LO.LlamaOracle({k_: v.double().numpy() for k_, v in w.items()}, SMALL.layers, SMALL.heads, SMALL.kv_heads,
+                         SMALL.head_dim, SMALL.rope_theta, SMALL.rms_eps, 16)
+    want = [orc.step(t) for t in toks]
+    gaps = []
+    for b in (1, 2, 4):
+        model.set_bits(b)
+        model.reset()
+        gap = 0.0
+        for t, ref in zip(toks, want):
+            model.token.fill_(t)
+            model.step_fused()
+            gap = max(gap, float(np.abs(model.logits[0].float().cpu().numpy() - ref).max() / np.abs(ref).max()))
+        gaps.append(gap)
+    print("logit gaps to the dense float64 decoder at 1, 2, 4 blocks:", gaps, flush=True)
+    assert gaps[0] > gaps[1] > gaps[2] and gaps[2] < 0.5 * gaps[0], gaps
+    full_logits = model.logits.clone()
+    # scores and configs, then the checkpoint with them, then a budgeted load
+    ids = torch.randint(0, SMALL.vocab, (2, 10), generator=torch.Generator().manual_seed(3))
+    scores = S.score_importance(model, ids, niter)
+    assert all(m.w_bit == niter for row in model.lin for m in row.values())
+    configs = S.compression_configs_for(model, scores)
+    model.save_checkpoint(str(tmp_path), compression_configs=configs, max_shard_bytes=300_000)
+    back = SyntheticLlamaDecoder.from_checkpoint(str(tmp_path), 16, dev(), niter=niter)
+    for t in toks:
+        back.token.fill_(t)
+        back.step_fused()
+    assert torch.equal(back.logits, full_logits)
+    mems = [c["memory"] for c in ck.read_compression_configs(str(tmp_path))]
+    budget = mems[len(mems) // 2]
+    cut = SyntheticLlamaDecoder.from_checkpoint(str(tmp_path), 16, dev(), max_memory_MB=budget / 1024 ** 2 + 1e-3)
+    assert cut.weight_bytes() <= budget < back.weight_bytes()
+    kept = {f"layer.{L}.{p}": m.w_bit for L, row in enumerate(cut.lin) for p, m in row.items()}
+    assert min(kept.values()) >= 1 and max(kept.values()) <= niter and len(set(kept.values())) > 1
+    for t in toks:
+        cut.token.fill_(t)
+        cut.step_fused()
+    assert torch.isfinite(cut.logits).all() and not torch.equal(cut.logits, full_logits)
