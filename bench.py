@@ -397,8 +397,8 @@ def main():
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     # HBM bytes per forward measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the largest launch of
     # that kernel (14336x4096, I=16), scaled by what the same counters read for a 256 MiB copy
-    # (FETCH_SIZE x2.0, WRITE_SIZE x1.0; profiles/gemv_traffic_counters.txt): 205 MB vs 126.9 MB algorithmic
-    traffic_ratio = 1.62
+    # (FETCH_SIZE x2.0, WRITE_SIZE x1.0; profiles/gemv_traffic_counters.txt): 146.6 MB vs 126.9 MB algorithmic
+    traffic_ratio = 1.16
 
     out = {
         "metric": "packed-sign GEMV HBM GB/s (decode sweep, Llama-3.1-8B linear shapes, T=1)",
@@ -417,7 +417,7 @@ def main():
                      "launches_per_step": dom_n,
                      "avg_us_per_launch": round(dom_ms * 1e3 / dom_n, 2),
                      "avg_algorithmic_bytes_per_launch": round(dom_bytes / dom_n),
-                     "traffic_note": "HBM bytes per launch = algorithmic x 1.62, the FETCH_SIZE+WRITE_SIZE ratio "
+                     "traffic_note": "HBM bytes per launch = algorithmic x 1.16, the FETCH_SIZE+WRITE_SIZE ratio "
                                      "measured on this kernel's largest launch (profiles/gemv_traffic_counters.txt)",
                      "whole_sweep_GBps_by_events": round(sweep_gbs, 1),
                      "best_layer": best},

@@ -145,12 +145,20 @@ struct Split {
 // the grid is cut into one run of workgroups per matrix, each with its own static
 // partition, partial-sum area and row count.
 constexpr int GEMV_MAX_GROUP = 4;
+constexpr int GEMV_WIDE_MIN_UNITS = 1024;   // 1024-row units from which one token runs on 16-wave workgroups
+constexpr int GEMV_PAIR_MIN_UNITS = 4;      // units per workgroup from which workgroups are paired
 struct GemvMat {
     const uint8_t *packed;
     const half_t *u, *vt;
     float *part;
     int M, row_tiles, kmax, first_wg;
     Split sp;
+    // 1: workgroups 2p and 2p + 1 share one range of (block, row tile, chunk PAIR) units and
+    // take the even / the odd 512-column chunk of every pair.  The two 64-byte halves of a
+    // 128-byte line of sign bytes are then requested at about the same time by neighbours on
+    // one XCD (the second request hits L2) instead of one unit apart by the same workgroup,
+    // by when the line has often been evicted and comes from HBM again.
+    int pair;
 };
 struct GemvGroup {
     GemvMat m[GEMV_MAX_GROUP];
@@ -158,10 +166,10 @@ struct GemvGroup {
 };
 
 template <int T, int WAVES, int R>
-__global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? (WAVES == 8 && R == 2 ? 4 : 2) : 1))) void gemv_kernel(
+__global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? (WAVES == 8 && R == 2 ? 4 : 2) : 1))) void gemv_kernel(
     const GemvGroup grp, const half_t *__restrict__ x, int N, int K, int n_chunks) {
     constexpr int RW = WAVES * R * 16;          // rows per workgroup
-    constexpr int COMBOS = 8 / WAVES;           // (jb, pg) producer combos per wave
+    constexpr int COMBOS = WAVES >= 8 ? 1 : 8 / WAVES;   // (jb, pg) producer combos per wave (waves 8.. of 16 have none)
     constexpr int ZHALVES = T * 16 * 4 * 16 * 8;   // one Z buffer
     constexpr int CSTEPS = 16 / WAVES;          // correction steps handled by each wave
     extern __shared__ __attribute__((aligned(16))) half_t lds[];
@@ -186,13 +194,16 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     for (int j = 1; j < GEMV_MAX_GROUP; j++)
         if (j < grp.n && wg >= grp.m[j].first_wg) mat = grp.m[j];
     wg -= mat.first_wg;
+    const int pair = mat.pair, cq = pair ? (wg & 1) : 0;      // chunk parity this workgroup takes
+    const int wv = wg >> pair;                                // its place in the partition
+    const int nch = n_chunks >> pair;                         // units per row of units
     const uint8_t *__restrict__ packed = mat.packed;
     const half_t *__restrict__ u = mat.u;
     const half_t *__restrict__ vt = mat.vt;
     float *__restrict__ part = mat.part;
     const int M = mat.M, row_tiles = mat.row_tiles, kmax = mat.kmax;
     const Split sp = mat.sp;
-    const int u_begin = sp.start(wg), u_end = sp.start(wg + 1);
+    const int u_begin = sp.start(wv), u_end = sp.start(wv + 1);
     if (u_begin >= u_end) return;
 
     const int64_t row_bytes = N >> 3;
@@ -235,6 +246,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     half8_t pv[COMBOS][2];        // vt pieces in flight for the next unit
     half8_t px[COMBOS][T][2];     // x pieces in flight for the next unit
     auto produce_issue = [&](int c) {
+        if (WAVES > 8 && wave >= 8) return;
 #pragma unroll
         for (int k = 0; k < COMBOS; k++) {
             const int combo = wave + k * WAVES, pg = combo & 3, jb = combo >> 2;
@@ -251,6 +263,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
         }
     };
     auto produce_write = [&](int buf) {
+        if (WAVES > 8 && wave >= 8) return;
         half_t *zbuf = zl + buf * ZHALVES;
 #pragma unroll
         for (int k = 0; k < COMBOS; k++) {
@@ -343,7 +356,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
             for (int t = 0; t < T; t++) *reinterpret_cast<float4_t *>(cx + (wave * T + t) * 16 + 4 * g) = corr[t];
         }
         __syncthreads();
-        const int slot = wg - sp.owner(rowid * n_chunks);
+        const int slot = ((wv - sp.owner(rowid * nch)) << pair) + cq;
 #pragma unroll
         for (int t = 0; t < T; t++) {
             float4_t cz = {0.f, 0.f, 0.f, 0.f};
@@ -363,16 +376,17 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     };
 
     // ---- pipeline fill: first unit's signs and Z -----------------------------
-    int rowid = u_begin / n_chunks, c = u_begin % n_chunks;
+    int rowid = u_begin / nch, c = u_begin % nch;
     set_row(rowid);
     uint4_t cur[R], nxt[R];
-    produce_issue(c);                               // first: Z production only waits for these
-    load_signs(cur, c);
+    auto chunk_of = [&](int unit_c) { return (unit_c << pair) + cq; };   // unit within its row -> 512-column chunk
+    produce_issue(chunk_of(c));                     // first: Z production only waits for these
+    load_signs(cur, chunk_of(c));
     uint32_t warm = 0;
     {
         // the flush after the last unit is not preceded by a crossing inside the loop:
         // pull the u rows it needs towards L2 now (value unused)
-        const int lrow = (u_end - 1) / n_chunks, fi = lrow / row_tiles, frt = lrow % row_tiles;
+        const int lrow = (u_end - 1) / nch, fi = lrow / row_tiles, frt = lrow % row_tiles;
         const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
         warm ^= *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
     }
@@ -382,7 +396,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
     // ---- steady state -------------------------------------------------------
     int buf = 0;
     for (int unit = u_begin; unit + 1 < u_end; unit++) {
-        const bool crossing = c + 1 == n_chunks;    // the next unit starts another row
+        const bool crossing = c + 1 == nch;         // the next unit starts another row
         const int cn = crossing ? 0 : c + 1;
         if (crossing) {
             // the row ends with this unit: pull its u rows towards L2 now (one
@@ -392,8 +406,8 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 4 && R == 4 ? 3 : 4
             warm ^= *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
             set_row(rowid + 1);                     // address arithmetic only
         }
-        produce_issue(cn);                          // L2-resident: first, so waiting for them does not wait for HBM
-        load_signs(nxt, cn);
+        produce_issue(chunk_of(cn));                // L2-resident: first, so waiting for them does not wait for HBM
+        load_signs(nxt, chunk_of(cn));
         __builtin_amdgcn_sched_barrier(0);          // keep the prefetch at the top of the unit
         consume(cur, buf);
         __builtin_amdgcn_sched_barrier(0);
@@ -430,6 +444,7 @@ struct RedMat {
     const half_t *bias;
     int I, M, row_tiles, kmax, y_off, first_block;
     Split sp;
+    int pair;       // as GemvMat::pair: two workgroups per place in the partition, slots 2k and 2k + 1
 };
 struct RedGroup {
     RedMat m[GEMV_MAX_GROUP];
@@ -487,9 +502,10 @@ __device__ __forceinline__ typename RedVec<VEC>::type slice_sum_any(const RedMat
 
 // nks[i] = workgroups whose unit range touched (block i, row tile rt) of this matrix
 __device__ __forceinline__ void count_partials(const RedMat &r, int rt, int n_chunks, int *nks) {
+    const int nch = n_chunks >> r.pair;
     for (int i = threadIdx.x; i < r.I; i += RED_OUT * RED_SL) {
-        const int first = (i * r.row_tiles + rt) * n_chunks;
-        nks[i] = r.sp.owner(first + n_chunks - 1) - r.sp.owner(first) + 1;
+        const int first = (i * r.row_tiles + rt) * nch;
+        nks[i] = (r.sp.owner(first + nch - 1) - r.sp.owner(first) + 1) << r.pair;
     }
 }
 
@@ -588,7 +604,7 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
 }
 
 struct Plan {
-    int waves, R, n_chunks, grid, n;
+    int waves, R, n_chunks, grid, n, pair;
     int row_tiles[GEMV_MAX_GROUP], kmax[GEMV_MAX_GROUP], first_wg[GEMV_MAX_GROUP];
     Split sp[GEMV_MAX_GROUP];
     int64_t part_off[GEMV_MAX_GROUP];      // in floats; part_off[n] = total
@@ -607,6 +623,7 @@ Plan make_plan(const int *I, const int *M, int n, int N, int T) {
     // to overlap sign decode and MFMA), four row tiles per wave (each Z fragment read
     // from LDS feeds four MFMAs per token) or two when the layer has too few units.
     const int cand1[4][3] = {{8, 4, 2}, {4, 4, 3}, {4, 2, 4}, {4, 1, 4}};
+    const int wide1[3] = {16, 4, 1};
     const int cand3[4][3] = {{8, 4, 1}, {8, 2, 1}, {4, 2, 1}, {4, 1, 1}};
     const int cand2[4][3] = {{8, 2, 2}, {4, 4, 2}, {4, 2, 2}, {4, 1, 2}};
     const int (*cand)[3] = T > 2 ? cand3 : T == 2 ? cand2 : cand1;
@@ -622,35 +639,72 @@ Plan make_plan(const int *I, const int *M, int n, int N, int T) {
         // enough units that every CU gets one
         if (tall && units >= 256) { pick = k; break; }
     }
-    p.waves = cand[pick][0];
-    p.R = cand[pick][1];
+    // One token, long stacks: one workgroup of 16 waves per CU.  Two 8-wave workgroups on a CU do
+    // not share it evenly (the older one is served first and finishes a third earlier, the
+    // younger one then runs on a half-empty CU); sixteen waves that meet at one barrier do.
+    const int *choice = cand[pick];
+    if (T == 1) {
+        bool tall = true;
+        int64_t units = 0;
+        for (int j = 0; j < n; j++) {
+            tall = tall && M[j] >= 1024;
+            units += bs_cdiv(M[j], 1024) * I[j] * p.n_chunks;
+        }
+        if (tall && units >= GEMV_WIDE_MIN_UNITS) choice = wide1;
+    }
+    p.waves = choice[0];
+    p.R = choice[1];
     int units[GEMV_MAX_GROUP], total = 0;
     for (int j = 0; j < n; j++) {
         p.row_tiles[j] = (int)bs_cdiv(M[j], p.waves * p.R * 16);
         units[j] = I[j] * p.row_tiles[j] * p.n_chunks;
         total += units[j];
     }
-    int grid = 256 * (T == 1 ? cand[pick][2] : T == 2 ? 2 : 1);
+    int grid = 256 * (T == 1 ? choice[2] : T == 2 ? 2 : 1);
     // prefer two units per workgroup (one pipeline fill amortised over two units) as
     // long as every CU still gets a workgroup
     if (grid > total / 2) grid = total / 2 >= 256 ? total / 2 : (total < 256 ? total : 256);
     if (grid < 1) grid = 1;
+    // Paired workgroups (GemvMat::pair) once a workgroup has several units to stream: the
+    // grid is then a multiple of 16, so that the contiguous run of workgroups an XCD gets
+    // starts and ends on a pair.
+    p.pair = (p.n_chunks % 2 == 0 && total >= GEMV_PAIR_MIN_UNITS * grid && grid >= 16 * n) ? 1 : 0;
+    int gj[GEMV_MAX_GROUP], sum = 0, biggest = 0;
+    for (int j = 0; j < n; j++) {
+        gj[j] = n == 1 ? grid : (int)(((int64_t)grid * units[j] + total / 2) / total);
+        if (p.pair) gj[j] &= ~1;
+        if (gj[j] < 1 + p.pair) gj[j] = 1 + p.pair;
+        if (gj[j] > units[j]) gj[j] = units[j];
+        sum += gj[j];
+        if (units[j] > units[biggest]) biggest = j;
+    }
+    if (p.pair) {
+        // round the grid to a multiple of 16 on the largest matrix (down when it can spare them)
+        const int over = sum % 16;
+        if (over && gj[biggest] > over + 16) gj[biggest] -= over;
+        else if (over && gj[biggest] + 16 - over <= units[biggest]) gj[biggest] += 16 - over;
+        else if (over) p.pair = 0;
+        if (!p.pair)      // back to the plain plan
+            for (int j = 0; j < n; j++) {
+                gj[j] = n == 1 ? grid : (int)(((int64_t)grid * units[j] + total / 2) / total);
+                if (gj[j] < 1) gj[j] = 1;
+                if (gj[j] > units[j]) gj[j] = units[j];
+            }
+    }
     int first = 0;
     int64_t off = 0;
     for (int j = 0; j < n; j++) {
-        int gj = n == 1 ? grid : (int)(((int64_t)grid * units[j] + total / 2) / total);
-        if (gj < 1) gj = 1;
-        if (gj > units[j]) gj = units[j];
+        const int places = gj[j] >> p.pair, uj = units[j] >> p.pair, nch = p.n_chunks >> p.pair;
         p.first_wg[j] = first;
-        first += gj;
-        p.sp[j].q = units[j] / gj;
-        p.sp[j].rem = units[j] % gj;
-        // most workgroups a row of n_chunks units can be spread over
-        int kmax = (int)bs_cdiv(p.n_chunks - 1, p.sp[j].q) + 1;
-        if (kmax > gj) kmax = gj;
-        p.kmax[j] = kmax;
+        first += gj[j];
+        p.sp[j].q = uj / places;
+        p.sp[j].rem = uj % places;
+        // most places a row of nch units can be spread over
+        int kmax = (int)bs_cdiv(nch - 1, p.sp[j].q) + 1;
+        if (kmax > places) kmax = places;
+        p.kmax[j] = kmax << p.pair;
         p.part_off[j] = off;
-        off += (int64_t)I[j] * kmax * T * M[j];
+        off += (int64_t)I[j] * p.kmax[j] * T * M[j];
     }
     p.grid = first;
     p.part_total = off;
@@ -677,6 +731,10 @@ int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int 
 
 template <int T>
 int launch_T(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
+    if (p.waves == 16) {
+        if constexpr (T == 1) return launch_one<T, 16, 4>(p, grp, x, N, K, s);
+        else return BS_ERR_SHAPE;
+    }
     if (p.waves == 8) {
         if constexpr (T == 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
         else if (p.R == 4) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
@@ -810,8 +868,9 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
     int y_off = 0, blocks = 0;
     for (int j = 0; j < a.n; j++) {
         g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
-                         p.first_wg[j], p.sp[j]};
-        r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks, p.sp[j]};
+                         p.first_wg[j], p.sp[j], p.pair};
+        r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks, p.sp[j],
+                        p.pair};
         y_off += a.M[j];
         if (mode != EPI_SWIGLU || j == 0) blocks += tp * (int)bs_cdiv(a.M[j], RED_OUT);
     }

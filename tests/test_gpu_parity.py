@@ -128,7 +128,9 @@ def oracle_refs(q, u, vt, x, bias=None):
 GEMV_CASES = [(1, 64, 512, 1), (2, 256, 512, 1), (4, 1024, 1024, 1), (3, 200, 1024, 2),
               (4, 4096, 4096, 1), (2, 1024, 4096, 4), (8, 4096, 4096, 4), (1, 1024, 4096, 1),
               (2, 14336, 4096, 1), (2, 4096, 14336, 1), (3, 512, 2048, 3), (2, 512, 1024, 5),
-              (2, 300, 1536, 6), (2, 256, 512, 7), (2, 512, 1024, 8), (16, 1024, 4096, 1)]
+              (2, 300, 1536, 6), (2, 256, 512, 7), (2, 512, 1024, 8), (16, 1024, 4096, 1),
+              # long stacks: 16-wave workgroups in pairs (one token), 8-wave pairs (two tokens)
+              (64, 2048, 4096, 1), (16, 4096, 4096, 2)]
 
 
 @pytest.mark.parametrize("I,M,N,T", GEMV_CASES)
@@ -139,7 +141,8 @@ def test_forward_decode_matches_oracle(I, M, N, T):
     y = IU.bitstack_forward_hip(q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())).cpu().numpy()
     assert y.dtype == np.float16 and y.shape == (T, M)
     assert_close(y, exact, "vs fp64")
-    assert_close(y, l0, "vs level-0 order")
+    if I <= 16:     # beyond that the level-0 order's own fp16 running sums are the larger error
+        assert_close(y, l0, "vs level-0 order")
 
 
 @pytest.mark.parametrize("I,M,N,T,K", [(2, 128, 512, 1, 16), (3, 256, 1024, 2, 5), (2, 64, 512, 1, 1)])
