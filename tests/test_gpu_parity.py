@@ -359,6 +359,49 @@ def test_decompose_on_gpu_matches_oracle():
     assert_close(y, want, "decomposed layer forward vs fp64")
 
 
+def test_single_layer_4096_decomposed_from_gaussian_weight():
+    """The reference's own CPU-runnable case at full size: W 4096 x 4096 fp32 ~ N(0, 0.02^2), seed 0,
+    four residual blocks of rank 16 (decomposed on the device), x 1 x 4096 fp16 ~ N(0, 1), all blocks
+    loaded; every fused level against the float64 closed form and against level 0."""
+    print("single layer 4096 x 4096, niter 4, k 16", flush=True)
+    M = N = 4096
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(M, N, generator=g) * 0.02
+    x = torch.randn(1, N, generator=g).half()
+    lin = torch.nn.Linear(N, M, bias=False)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        mod = BitStackLinear.from_linear(lin.to(dev()), w_bit=4, k=16, bias=False, fused_level=0, name="single")
+    q = np.stack([getattr(mod, f"qweight_{i}").cpu().numpy() for i in range(4)])
+    u = np.stack([getattr(mod, f"u_{i}").cpu().numpy() for i in range(4)])
+    vt = np.stack([getattr(mod, f"vt_{i}").cpu().numpy() for i in range(4)])
+    wn = w.numpy()
+    # block 0 holds the signs of W itself, bit for bit; its product is the best rank-16 fit of |W|
+    assert np.array_equal(q[0], O.pack_sign(np.where(wn >= 0, 1, -1).astype(np.int8)))
+    uu, sv, vv = np.linalg.svd(np.abs(wn).astype(np.float64), full_matrices=False)
+    best = (uu[:, :16] * sv[:16]) @ vv[:16]
+    assert np.abs(u[0].astype(np.float64) @ vt[0].astype(np.float64) - best).max() <= 4e-3 * np.abs(best).max()
+    # the approximation error falls with every block loaded
+    errs = [float(np.linalg.norm(O.reconstruct_w_exact(q[:b], u[:b], vt[:b]) - wn) / np.linalg.norm(wn)) for b in (1, 2, 3, 4)]
+    print("relative error of the rebuilt weight with 1..4 blocks:", [round(e, 4) for e in errs], flush=True)
+    assert errs[0] > errs[1] > errs[2] > errs[3] and errs[0] < 0.65 and errs[3] < 0.2
+    exact = x.double().numpy() @ O.reconstruct_w_exact(q, u, vt).T
+    xd = x.to(dev())
+    y0 = mod(xd)                                        # level 0: torch ops, fp16 sums
+    assert_close(y0.cpu().numpy(), exact, "level 0 vs fp64")
+    mod.stack_blocks()
+    for level in (1, 2, 3, 4, 5):
+        mod.fused_level = level
+        y = mod(xd.view(1, 1, N)).view(1, M)
+        assert_close(y.cpu().numpy(), exact, f"level {level} vs fp64")
+        assert_close(y.cpu().numpy(), y0.cpu().numpy(), f"level {level} vs level 0")
+    # and the layer does what the dense one did, to the accuracy four blocks give
+    dense = x.double().numpy() @ wn.astype(np.float64).T
+    mx, mn = rel_errors(y.cpu().numpy(), dense)
+    print(f"level 5 vs the dense layer: max_rel={mx:.3f} mean_rel={mn:.3f}", flush=True)
+    assert mn < 0.3
+
+
 # ------------------------------------------------------------- seeded random shapes
 def _random_cases(n, seed):
     rng = np.random.default_rng(seed)
