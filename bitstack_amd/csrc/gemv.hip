@@ -382,19 +382,21 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
     auto chunk_of = [&](int unit_c) { return (unit_c << pair) + cq; };   // unit within its row -> 512-column chunk
     produce_issue(chunk_of(c));                     // first: Z production only waits for these
     load_signs(cur, chunk_of(c));
-    uint32_t warm = 0;
+    uint32_t warm0;      // loaded for its side effect only (the line ends up in L2)
     {
         // the flush after the last unit is not preceded by a crossing inside the loop:
         // pull the u rows it needs towards L2 now (value unused)
         const int lrow = (u_end - 1) / nch, fi = lrow / row_tiles, frt = lrow % row_tiles;
         const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
-        warm ^= *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
+        warm0 = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
     }
     produce_write(0);
     __syncthreads();
+    asm volatile("" ::"v"(warm0));                  // keeps the load; by now it has long arrived
 
     // ---- steady state -------------------------------------------------------
     int buf = 0;
+    uint32_t warm_in = 0;
     for (int unit = u_begin; unit + 1 < u_end; unit++) {
         const bool crossing = c + 1 == nch;         // the next unit starts another row
         const int cn = crossing ? 0 : c + 1;
@@ -403,7 +405,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
             // dword per row, value unused) so the flush below does not wait on HBM
             const int fi = rowid / row_tiles, frt = rowid % row_tiles;
             const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
-            warm ^= *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
+            warm_in = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
             set_row(rowid + 1);                     // address arithmetic only
         }
         produce_issue(chunk_of(cn));                // L2-resident: first, so waiting for them does not wait for HBM
@@ -411,6 +413,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
         __builtin_amdgcn_sched_barrier(0);          // keep the prefetch at the top of the unit
         consume(cur, buf);
         __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::"v"(warm_in));              // keeps the load alive; waited for only here, behind the MFMA loop
         produce_write(buf ^ 1);
         __syncthreads();
         if (crossing) {
@@ -425,7 +428,6 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
     // ---- drain: last unit, nothing left to prefetch -----------------------------
     consume(cur, buf);
     flush(rowid);
-    if (warm == 0x9e3779b9u && part == nullptr) part[0] = 0.f;   // keeps the warm-up loads alive
 }
 
 // y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ) where k
