@@ -451,6 +451,12 @@ def main():
 
     if not a.no_extras:
         out["decode_8b"] = e2e_decode(torch, dev)
+        torch.cuda.empty_cache()
+        # 70B shape: batch 8 with 2048-token prompts (one-pass prefill, strip kernel), then batch 1 (GEMV)
+        out["decode_70b"] = e2e_decode_70b(torch, dev, batch=8, prompt_len=2048)
+        torch.cuda.empty_cache()
+        out["decode_70b_batch1"] = e2e_decode_70b(torch, dev, batch=1, prompt_len=16)
+        torch.cuda.empty_cache()
 
     if not a.no_cpu_baseline:
         # bounded sample of the same sweep: every shape, blocks {1, 2, 4} (7/31 of the pass)
