@@ -251,6 +251,20 @@ class SyntheticLlamaDecoder:
                 m.set_bit(b)
         self._groups = None
 
+    def set_memory_budget(self, path, max_memory_MB=None, compression_config=None):
+        """Move the loaded decoder to another size of the same checkpoint while it runs: the
+        config that fits max_memory_MB (bitstack/utils/model_utils.py:179-187) or the one given;
+        linears that get fewer blocks free the surplus, those that get more read only the
+        missing blocks from `path` (checkpoint.apply_compression_config).  The KV cache and
+        the position stay as they are.  Returns (bytes_freed, bytes_loaded)."""
+        from bitstack_amd.utils import checkpoint as ck
+        if compression_config is None:
+            compression_config = ck.retrieve_compression_config(ck.read_compression_configs(path), max_memory_MB)
+        linears = {f"layer.{L}.{p}": m for L, row in enumerate(self.lin) for p, m in row.items()}
+        moved = ck.apply_compression_config(path, linears, compression_config)
+        self._groups = None
+        return moved
+
     def reset(self):
         self.pos.zero_()
         self.kcache.zero_()

@@ -507,3 +507,20 @@ def test_whole_flow_dense_to_compressed_to_budgeted_decoder(tmp_path):
         cut.token.fill_(t)
         cut.step_fused()
     assert torch.isfinite(cut.logits).all() and not torch.equal(cut.logits, full_logits)
+    # the running full-size decoder shrunk to that budget (blocks freed) is the decoder loaded at
+    # it, and grown back (blocks read from disk) it is the full one again
+    full_bytes = back.weight_bytes()
+    freed, loaded = back.set_memory_budget(str(tmp_path), max_memory_MB=budget / 1024 ** 2 + 1e-3)
+    assert freed > 0 and loaded == 0 and back.weight_bytes() == cut.weight_bytes() == full_bytes - freed
+    back.reset()
+    for t in toks:
+        back.token.fill_(t)
+        back.step_fused()
+    assert torch.equal(back.logits, cut.logits)
+    freed2, loaded2 = back.set_memory_budget(str(tmp_path), compression_config={k_: niter for k_ in kept})
+    assert freed2 == 0 and loaded2 == freed and back.weight_bytes() == full_bytes
+    back.reset()
+    for t in toks:
+        back.token.fill_(t)
+        back.step_fused()
+    assert torch.equal(back.logits, full_logits)
