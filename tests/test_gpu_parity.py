@@ -112,6 +112,32 @@ def test_reconstruct_w_matches_oracle(I, M, N, K):
     assert np.array_equal(got2.view(np.uint16), got.view(np.uint16))
 
 
+def test_reference_self_check_scenario():
+    """The one numeric check the reference carries (bitstack/utils/inference_utils.py:597-626):
+    M = N = 32, k = 16, one block, sign / u / vt / x drawn from N(0, 1) in fp16; the rebuilt weight
+    against `(sign * matmul(u, vt)).sum(0)` within atol = 1e-2, rtol = 0 — and, from the lines it
+    keeps commented out, the fused forward against `x @ W.T`."""
+    g = torch.Generator().manual_seed(0)
+    M = N = 32
+    x = torch.randn(1, 1, N, generator=g).half()
+    sign = torch.sign(torch.randn(1, M, N, generator=g).half())
+    sign[sign == 0] = 1
+    packed = torch.from_numpy(O.pack_sign(sign.to(torch.int8).numpy().reshape(-1))).reshape(1, -1)
+    u = torch.randn(1, M, 16, generator=g).half()
+    vt = torch.randn(1, 16, N, generator=g).half()
+    ref_w = (sign * torch.matmul(u.float(), vt.float()).half()).sum(dim=0)           # the script's torch_output
+    pd, ud, vd = packed.to(dev()), u.to(dev()), vt.to(dev())
+    w = IU.unpack_and_reconstruct_w_hip(pd, ud, vd).cpu()
+    assert torch.allclose(w, ref_w, atol=1e-2, rtol=0)
+    w2 = IU.reconstruct_w_hip(sign.to(torch.int8).to(dev()), ud, vd).cpu()
+    assert torch.equal(w2, w)
+    exact_w = O.reconstruct_w_exact(packed.numpy(), u.numpy(), vt.numpy())
+    assert np.all(np.abs(w.double().numpy() - exact_w) <= np.spacing(np.abs(exact_w).astype(np.float16)).astype(np.float64))
+    y = IU.bitstack_forward_hip(pd, ud, vd, x.to(dev())).cpu()
+    assert tuple(y.shape) == (1, 1, M)
+    assert_close(y.view(1, M).numpy(), x.view(1, N).double().numpy() @ exact_w.T, "forward vs fp64")
+
+
 def test_reconstruct_zero_blocks_is_zero():
     q, u, vt, _ = synthetic_layer(64, 128, 2, 1, device=dev())
     w = IU.unpack_and_reconstruct_w_hip(q[:0], u[:0], vt[:0])
