@@ -156,7 +156,9 @@ GEMV_CASES = [(1, 64, 512, 1), (2, 256, 512, 1), (4, 1024, 1024, 1), (3, 200, 10
               (2, 14336, 4096, 1), (2, 4096, 14336, 1), (3, 512, 2048, 3), (2, 512, 1024, 5),
               (2, 300, 1536, 6), (2, 256, 512, 7), (2, 512, 1024, 8), (16, 1024, 4096, 1),
               # long stacks: 16-wave workgroups in pairs (one token), 8-wave pairs (two tokens)
-              (64, 2048, 4096, 1), (16, 4096, 4096, 2)]
+              (64, 2048, 4096, 1), (16, 4096, 4096, 2),
+              # 16 waves with a ragged last row tile; 16 waves, odd chunk count (no pairing)
+              (48, 2500, 4096, 1), (200, 1100, 1536, 1)]
 
 
 @pytest.mark.parametrize("I,M,N,T", GEMV_CASES)
