@@ -47,7 +47,9 @@ def make_group(shapes, N, T, seed, bias=False):
 GROUP_CASES = [([(3, 512), (5, 128), (2, 128)], 512, 1), ([(3, 4096), (5, 1024), (2, 1024)], 4096, 1),
                ([(2, 1024), (4, 256)], 1024, 2), ([(1, 300), (2, 77), (3, 64), (1, 512)], 1536, 3),
                ([(2, 512), (3, 256)], 1024, 4), ([(2, 512), (1, 256)], 512, 5), ([(2, 256), (2, 256)], 1024, 8),
-               ([(2, 300), (3, 77), (1, 64)], 1536, 9), ([(3, 1024), (2, 256)], 4096, 16), ([(2, 200), (2, 200)], 384, 32), ([(2, 300), (1, 64)], 640, 48)]
+               ([(2, 300), (3, 77), (1, 64)], 1536, 9), ([(3, 1024), (2, 256)], 4096, 16), ([(2, 200), (2, 200)], 384, 32), ([(2, 300), (1, 64)], 640, 48),
+               # long stacks: 16-wave workgroups in pairs, the grid cut into even runs per matrix
+               ([(32, 2048), (30, 1024), (34, 1100)], 4096, 1), ([(20, 4096), (12, 1024)], 4096, 2)]
 
 
 @pytest.mark.parametrize("shapes,N,T", GROUP_CASES)
