@@ -129,3 +129,30 @@ def test_group_and_decode_step_validation(L):
     assert att(one, one, one, one, one, one, one, 1, 32, 8, 128, 10000, nul) == -2              # max_len
     assert att(one, one, one, one, one, nul, one, 1, 32, 8, 128, 128, nul) == -1                # pos
     assert att(one, odd, one, one, one, one, one, 1, 32, 8, 128, 128, nul) == -4
+
+
+def test_no_fallback_when_the_library_or_the_device_is_missing(tmp_path):
+    """The product path fails loudly: a missing shared library is an error that names the
+    build step, and the HIP entry points refuse host tensors (only fused_level 0 is torch-only)."""
+    import subprocess
+    import sys
+    import torch
+    from bitstack_amd import BitStackLinear
+    from bitstack_amd.utils import inference_utils as IU
+    from bitstack_amd.utils import pack_utils as PU
+    code = ("import bitstack_amd._lib as L\n"
+            "try:\n    L.lib()\nexcept RuntimeError as e:\n    print('RAISED', e)\n")
+    env = dict(os.environ, BITSTACK_AMD_LIB=str(tmp_path / "absent.so"))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env,
+                         cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert "RAISED" in out.stdout and "is missing" in out.stdout and "no fallback" in out.stdout, out.stdout + out.stderr
+    q = torch.zeros(2, 64 * 512 // 8, dtype=torch.uint8)
+    u, vt, x = torch.zeros(2, 64, 16).half(), torch.zeros(2, 16, 512).half(), torch.zeros(1, 512).half()
+    for call in (lambda: IU.bitstack_forward_hip(q, u, vt, x), lambda: IU.unpack_and_reconstruct_w_hip(q, u, vt),
+                 lambda: PU.unpack_sign_hip(q[0], (64, 512)), lambda: IU.linear_f16_hip(x, torch.zeros(64, 512).half())):
+        with pytest.raises(RuntimeError, match="HIP device"):
+            call()
+    mod = BitStackLinear(2, 512, 64, 16, False, False, "cpu", fused_level=5)
+    mod.stack_blocks()
+    with pytest.raises(RuntimeError, match="HIP device"):
+        mod(x)
