@@ -693,6 +693,13 @@ Plan make_plan(const int *I, const int *M, int n, int N, int T) {
                 if (gj[j] > units[j]) gj[j] = units[j];
             }
     }
+    if (!p.pair && n > 1) {
+        // rounding per matrix may leave one workgroup too many: it would wait for a free slot
+        // and run after the others (a launch of 513 takes a fifth longer than one of 512)
+        sum = 0;
+        for (int j = 0; j < n; j++) sum += gj[j];
+        while (sum > grid && gj[biggest] > 1) { gj[biggest]--; sum--; }
+    }
     int first = 0;
     int64_t off = 0;
     for (int j = 0; j < n; j++) {
