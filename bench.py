@@ -419,6 +419,10 @@ def main():
                      "avg_algorithmic_bytes_per_launch": round(dom_bytes / dom_n),
                      "traffic_note": "HBM bytes per launch = algorithmic x 1.16, the FETCH_SIZE+WRITE_SIZE ratio "
                                      "measured on this kernel's largest launch (profiles/gemv_traffic_counters.txt)",
+                     "limiter": "instruction issue, not HBM: the contraction is 16 MACs per sign bit on MFMA plus one VALU merge "
+                                "per 128 signs; counters show 6.4 VALU per MFMA and the loop runs at the rate a stand-alone "
+                                "v_and_or_b32 + MFMA loop of that mix measures (about 3.3 TB/s of sign bytes); below 10 MB per "
+                                "layer the two launches' fixed cost (about 8 us) dominates",
                      "whole_sweep_GBps_by_events": round(sweep_gbs, 1),
                      "best_layer": best},
     }
