@@ -44,6 +44,14 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// LDS rows of a k-step.  GK = 32: 64-byte rows with no padding, the four 16-byte pieces of a
+// row XOR-ed with bits 2..3 of the row number - staging writes (four lanes per row, rows 64 bytes
+// apart) and fragment reads (sixteen rows, one piece each) then both spread over all banks;
+// with padded rows the writes of the 256 x 256 kernel conflicted (SQ_LDS_BANK_CONFLICT about a
+// tenth of its cycles).  Wider steps: rows padded by 8 halves (no conflicts measured).
+__host__ __device__ constexpr bool lds_swizzled(int gk) { return gk == 32; }
+__host__ __device__ constexpr int lds_stride(int gk) { return lds_swizzled(gk) ? gk : gk + 8; }
+
 template <int WT, int WF, int AT, int AF, int GK, bool KTAIL>
 __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     const half_t *__restrict__ x, const half_t *__restrict__ w, const half_t *__restrict__ bias,
@@ -52,12 +60,13 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     constexpr int BT = WT * AT * 32, BF = WF * AF * 32;      // workgroup tile: tokens x features
     constexpr int ROWS = BT + BF;                            // LDS rows per buffer (x rows, then w rows)
     constexpr int PPR = GK / 8;                              // 16-byte pieces per row and k-step
-    constexpr int LSTRIDE = GK + 8;                          // halves per LDS row (padded)
+    constexpr int LSTRIDE = lds_stride(GK);                  // halves per LDS row
+    constexpr bool SWZ = lds_swizzled(GK);
     constexpr int JX = BT * PPR / THREADS, JW = BF * PPR / THREADS;   // pieces per thread: x rows, w rows
     static_assert(BT * PPR % THREADS == 0 && BF * PPR % THREADS == 0, "every thread stages whole pieces");
     constexpr int PER_THREAD = JX + JW;
     extern __shared__ __attribute__((aligned(16))) half_t lds_raw[];
-    half_t (*lds)[ROWS * (GK + 8)] = reinterpret_cast<half_t (*)[ROWS * (GK + 8)]>(lds_raw);
+    half_t (*lds)[ROWS * LSTRIDE] = reinterpret_cast<half_t (*)[ROWS * LSTRIDE]>(lds_raw);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = blockIdx.y * BT, m0 = blockIdx.x * BF;
@@ -80,7 +89,7 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
         const int r = lrow + (THREADS / PPR) * (isx ? j : j - JX);
         const int rr = isx ? min(r, T - 1 - t0) : min(r, M - 1 - m0);
         off[j] = (uint32_t)rr * (uint32_t)N * 2u + 16u * lpiece;
-        dst[j] = ((isx ? 0 : BT) + r) * LSTRIDE + 8 * lpiece;
+        dst[j] = ((isx ? 0 : BT) + r) * LSTRIDE + 8 * (SWZ ? (lpiece ^ ((r >> 2) & 3)) : lpiece);
     }
 
     float16_t acc[AT][AF];
@@ -134,15 +143,16 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     constexpr int NK = GK / 16;
     static_assert(NK % 2 == 0, "the fragment sets alternate with a period of two sub-steps");
     half8_t fa[2][AT], fb[2][AF];
+    const int swz = (l32 >> 2) & 3;             // wt, wf and the tile offsets are multiples of 32: only the lane's row counts
     auto load_frags = [&](auto setc, int buf, int kk) {
         constexpr int set = decltype(setc)::value;
         const half_t *xs = &lds[buf][0], *ws = &lds[buf][BT * LSTRIDE];
 #pragma unroll
         for (int j = 0; j < AT; j++)
-            fa[set][j] = *reinterpret_cast<const half8_t *>(xs + (wt + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
+            fa[set][j] = *reinterpret_cast<const half8_t *>(xs + (wt + 32 * j + l32) * LSTRIDE + (SWZ ? 8 * ((2 * kk + kh) ^ swz) : 16 * kk + 8 * kh));
 #pragma unroll
         for (int j = 0; j < AF; j++)
-            fb[set][j] = *reinterpret_cast<const half8_t *>(ws + (wf + 32 * j + l32) * LSTRIDE + 16 * kk + 8 * kh);
+            fb[set][j] = *reinterpret_cast<const half8_t *>(ws + (wf + 32 * j + l32) * LSTRIDE + (SWZ ? 8 * ((2 * kk + kh) ^ swz) : 16 * kk + 8 * kh));
     };
     auto mfmas = [&](auto setc) {
         constexpr int set = decltype(setc)::value;
@@ -311,7 +321,7 @@ template <int WT, int WF, int AT, int AF, int GK>
 int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y, int T, int M, int N,
                  hipStream_t s) {
     constexpr int BT = WT * AT * 32, BF = WF * AF * 32;
-    constexpr size_t lds = (size_t)2 * (BT + BF) * (GK + 8) * sizeof(half_t);
+    constexpr size_t lds = (size_t)2 * (BT + BF) * lds_stride(GK) * sizeof(half_t);
     static size_t granted[2][BS_MAX_DEVICES] = {};
     int st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>, lds, granted[0]);
     if (st == BS_OK) st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>, lds, granted[1]);
