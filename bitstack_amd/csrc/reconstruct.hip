@@ -80,9 +80,22 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                 sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
             }
         };
-        half4_t b_cur, b_nxt;
-        uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
-        if (row_begin + wave * 16 < row_end) load_block(i0, min(row_begin + wave * 16 + lm, M - 1), b_cur, sw_cur);
+        // The (row step, block) pairs of this wave form one sequence; its loads run TWO pairs
+        // ahead (one pair of work does not cover the memory latency: the waves were waiting
+        // for data two thirds of their time).
+        half4_t b_cur, b_n1, b_n2;
+        uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+        const int first_row = row_begin + wave * 16;
+        // Requests are unconditional (behind the last pair they repeat its row step): a
+        // branch around a load makes the compiler wait for every load in flight at the join.
+        const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
+        int pf_i = 0, pf_m0 = first_row;           // the pair the next request is for
+        auto request = [&](half4_t &b, uint4_t &sw) {
+            load_block(i0 + pf_i, min(min(pf_m0, last_m0) + lm, M - 1), b, sw);
+            if (++pf_i == ib) { pf_i = 0; pf_m0 += 64; }
+        };
+        request(b_cur, sw_cur);
+        request(b_n1, sw_n1);
 
         // four blocks at a time, so that their loads are in flight together
         for (int q0 = 0; q0 < ib; q0 += 4) {
@@ -111,15 +124,21 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
             for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
             for (int i = 0; i < ib; i++) {
-                if (i + 1 < ib) load_block(i0 + i + 1, row, b_nxt, sw_nxt);
-                else if (m0 + 64 < row_end) load_block(i0, min(m0 + 64 + lm, M - 1), b_nxt, sw_nxt);
+                request(b_n2, sw_n2);
                 const uint4_t swc = sw_cur;      // bit 1 means +1: the product enters negated, times -1.0f
                 const half_t *vb = vl + i * VBLOCK + aoff;
+                // all eight fragments first, and every product one patch ahead of the sign FMAs
+                // that use it: neither the LDS nor the MFMA latency sits in front of them
+                half4_t a[8];
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
+                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
-                    const half_t *ap = vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD;
-                    const half4_t a = *reinterpret_cast<const half4_t *>(ap);
-                    float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float4_t p = p_next;
+                    if (s + 1 < 8)
+                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     if (PACKED) {
                         uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
 #pragma unroll
@@ -137,8 +156,10 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                         }
                     }
                 }
-                b_cur = b_nxt;
-                sw_cur = sw_nxt;
+                b_cur = b_n1;
+                sw_cur = sw_n1;
+                b_n1 = b_n2;
+                sw_n1 = sw_n2;
             }
 
             if (m0 + lm < M) {

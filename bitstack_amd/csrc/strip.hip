@@ -108,9 +108,24 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
         }
         sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + ((n0 + q * SF_COLS) >> 3));
     };
-    half4_t b_cur, b_nxt;
-    uint4_t sw_cur = {0, 0, 0, 0}, sw_nxt = {0, 0, 0, 0};
-    if (row_begin + wave * 16 < row_end) load_block(0, min(row_begin + wave * 16 + lm, M - 1), 0, b_cur, sw_cur);
+    // The (row step, strip, block) triples of this wave form one sequence; its sign and u loads run
+    // TWO triples ahead, and they are unconditional (behind the last triple they repeat its row
+    // step): a branch around a load makes the compiler wait for every load in flight at the join,
+    // which left the waves waiting for data half of their time.
+    half4_t b_cur, b_n1, b_n2;
+    uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+    const int first_row = row_begin + wave * 16;
+    const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
+    int pf_i = 0, pf_q = 0, pf_m0 = first_row;      // the triple the next request is for
+    auto request = [&](half4_t &b, uint4_t &sw) {
+        load_block(pf_i, min(min(pf_m0, last_m0) + lm, M - 1), pf_q, b, sw);
+        if (++pf_i == I) {
+            pf_i = 0;
+            if (++pf_q == ns) { pf_q = 0; pf_m0 += 64; }
+        }
+    };
+    request(b_cur, sw_cur);
+    request(b_n1, sw_n1);
 
     // x image: token rows beyond T are zero
     for (int idx = tid; idx < TT * 16 * ns * 16; idx += 256) {
@@ -159,7 +174,6 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
     const half_t *xfrag = xl + lm * xstride + 8 * g;
 
     for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += 64) {
-        const int row = min(m0 + lm, M - 1);
         float4_t yacc[TT];
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -170,17 +184,20 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
             for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
             for (int i = 0; i < I; i++) {
-                // signs and u one block ahead, across strips and row steps
-                if (i + 1 < I) load_block(i + 1, row, q, b_nxt, sw_nxt);
-                else if (q + 1 < ns) load_block(0, row, q + 1, b_nxt, sw_nxt);
-                else if (m0 + 64 < row_end) load_block(0, min(m0 + 64 + lm, M - 1), 0, b_nxt, sw_nxt);
+                request(b_n2, sw_n2);
                 const uint4_t swc = sw_cur;         // bit 1 means +1: the product enters negated, times -1.0f
                 const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
+                // all eight fragments first, and every product one patch ahead of the sign FMAs that use it
+                half4_t a[8];
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
+                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
-                    const half_t *ap = vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD;
-                    const half4_t a = *reinterpret_cast<const half4_t *>(ap);
-                    const float4_t p = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float4_t p = p_next;
+                    if (s + 1 < 8)
+                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     const uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
@@ -188,8 +205,10 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
                         acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
                     }
                 }
-                b_cur = b_nxt;
-                sw_cur = sw_nxt;
+                b_cur = b_n1;
+                sw_cur = sw_n1;
+                b_n1 = b_n2;
+                sw_n1 = sw_n2;
             }
 
             // y[token, row] of this strip: D[token 4g + v, row lm] = sum_k x[token, col(k)] * w[row, col(k)]
