@@ -68,8 +68,12 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         // u rows and sign words of one (row step, block); requested one block ahead, also
         // across the end of a row step (first block of the next 16 rows), and issued for
         // the very first block before the vt strip is staged
-        auto load_block = [&](int i, int row, half4_t &b, uint4_t &sw) {
-            const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+        // Addresses are a wave-uniform 64-bit base (the block: scalar arithmetic) plus a 32-bit
+        // offset per lane that depends on the row only and is renewed once per row step.
+        uint32_t off_u, off_s;                      // bytes: this lane's u row (its four ranks) and sign row
+        auto load_block = [&](int i, half4_t &b, uint4_t &sw) {
+            const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
+            const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
             if (K == 16) {
                 b = *reinterpret_cast<const half4_t *>(up);
             } else {
@@ -77,7 +81,8 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                 for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
             }
             if (PACKED) {
-                sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + (n0 >> 3));
+                const uint8_t *sb = packed + i * block_bytes + (n0 >> 3);
+                sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
             }
         };
         // The (row step, block) pairs of this wave form one sequence; its loads run TWO pairs
@@ -90,9 +95,19 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         // branch around a load makes the compiler wait for every load in flight at the join.
         const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
         int pf_i = 0, pf_m0 = first_row;           // the pair the next request is for
+        auto set_row = [&](int m0) {
+            const int row = min(min(m0, last_m0) + lm, M - 1);
+            off_u = (uint32_t)(row * K + 4 * g) * 2u;
+            off_s = (uint32_t)row * (uint32_t)row_bytes;
+        };
+        set_row(pf_m0);
         auto request = [&](half4_t &b, uint4_t &sw) {
-            load_block(i0 + pf_i, min(min(pf_m0, last_m0) + lm, M - 1), b, sw);
-            if (++pf_i == ib) { pf_i = 0; pf_m0 += 64; }
+            load_block(i0 + pf_i, b, sw);
+            if (++pf_i == ib) {
+                pf_i = 0;
+                pf_m0 += 64;
+                set_row(pf_m0);
+            }
         };
         request(b_cur, sw_cur);
         request(b_n1, sw_n1);
@@ -208,7 +223,9 @@ __global__ __launch_bounds__(256) void reconstruct_generic_kernel(
 template <bool PACKED>
 int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *u, const half_t *vt,
                        half_t *w, int I, int M, int N, int K, hipStream_t s) {
-    const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && bs_aligned(vt, 16) && bs_aligned(w, 16) &&
+    // the tiled kernel addresses a block's u and sign rows with 32-bit byte offsets
+    const bool small = (int64_t)M * (N >> 3) < ((int64_t)1 << 32) && (int64_t)M * K * 2 < ((int64_t)1 << 32);
+    const bool tiled = (N % RT_COLS == 0) && I >= 1 && I <= RT_MAXB && small && bs_aligned(vt, 16) && bs_aligned(w, 16) &&
                        bs_aligned(u, 8) && (PACKED ? bs_aligned(packed, 16) : bs_aligned(sign, 4));
     if (tiled) {
         // One wave of workgroups: as many row groups as the resident slots allow (LDS decides

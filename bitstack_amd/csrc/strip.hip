@@ -98,15 +98,28 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
     const int acol = 8 * (lm >> 2) + (lm & 3);
     const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
 
-    auto load_block = [&](int i, int row, int q, half4_t &b, uint4_t &sw) {
-        const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+    const int first_row = row_begin + wave * 16;
+    const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
+    // Addresses are a wave-uniform 64-bit base (block, strip: scalar arithmetic) plus a 32-bit
+    // offset per lane that depends on the row only and is renewed once per row step; worked out
+    // per request in 64 bits per lane, the multiplications were a fifth of the kernel's VALU time.
+    uint32_t off_u, off_s;                          // bytes: this lane's u row (its four ranks) and sign row
+    auto set_row = [&](int m0) {
+        const int row = min(min(m0, last_m0) + lm, M - 1);
+        off_u = (uint32_t)(row * K + 4 * g) * 2u;
+        off_s = (uint32_t)row * (uint32_t)row_bytes;
+    };
+    auto load_block = [&](int i, int q, half4_t &b, uint4_t &sw) {
+        const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
+        const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
         if (K == 16) {
             b = *reinterpret_cast<const half4_t *>(up);
         } else {
 #pragma unroll
             for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
         }
-        sw = *reinterpret_cast<const uint4_t *>(packed + i * block_bytes + row * row_bytes + ((n0 + q * SF_COLS) >> 3));
+        const uint8_t *sb = packed + i * block_bytes + ((n0 + q * SF_COLS) >> 3);
+        sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
     };
     // The (row step, strip, block) triples of this wave form one sequence; its sign and u loads run
     // TWO triples ahead, and they are unconditional (behind the last triple they repeat its row
@@ -114,14 +127,17 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
     // which left the waves waiting for data half of their time.
     half4_t b_cur, b_n1, b_n2;
     uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
-    const int first_row = row_begin + wave * 16;
-    const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
     int pf_i = 0, pf_q = 0, pf_m0 = first_row;      // the triple the next request is for
+    set_row(pf_m0);
     auto request = [&](half4_t &b, uint4_t &sw) {
-        load_block(pf_i, min(min(pf_m0, last_m0) + lm, M - 1), pf_q, b, sw);
+        load_block(pf_i, pf_q, b, sw);
         if (++pf_i == I) {
             pf_i = 0;
-            if (++pf_q == ns) { pf_q = 0; pf_m0 += 64; }
+            if (++pf_q == ns) {
+                pf_q = 0;
+                pf_m0 += 64;
+                set_row(pf_m0);
+            }
         }
     };
     request(b_cur, sw_cur);
