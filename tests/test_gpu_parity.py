@@ -346,6 +346,35 @@ def test_module_levels_agree_with_level0(bias):
         mod(xd)
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_empty_and_ragged_inputs(bias):
+    """No tokens, no blocks, odd leading dimensions: the shapes torch's F.linear accepts at level 0
+    (BitStackLinear.py:105-114) give the same shapes and values at every level."""
+    M, N, I = 96, 512, 3
+    mod, x = build_module(M, N, I, bias, 23)
+    mod = mod.to(dev())
+    xd = x.to(dev())
+    for level in (0, 1, 2, 3, 4, 5):
+        mod.fused_level = level
+        mod.set_bit(I)
+        if level == 1:
+            mod.stack_blocks()                          # level 0 reads the per-block buffers, the others the stacked ones
+        for shape in ((0, N), (2, 0, N), (0, 3, N)):
+            y = mod(torch.empty(shape, dtype=torch.float16, device=dev()))
+            assert y.dtype == torch.float16 and tuple(y.shape) == shape[:-1] + (M,)
+        # 1 x 1 x N and 5 x 1 x N: one token and five may run different kernels, same numbers up to the rounding points
+        y1 = mod(xd[:1].view(1, 1, N))
+        assert tuple(y1.shape) == (1, 1, M)
+        y5 = mod(xd.repeat(2, 1)[:5].view(5, 1, N))
+        assert tuple(y5.shape) == (5, 1, M)
+        assert float((y5[0, 0].float() - y1[0, 0].float()).abs().max()) <= 4e-3 * float(y1.float().abs().max())
+        # no blocks at all: w = 0, the output is the bias (or zero)
+        mod.set_bit(0)
+        y = mod(xd)
+        want = mod.bias.expand(3, M) if bias else torch.zeros(3, M, dtype=torch.float16, device=dev())
+        assert torch.equal(y, want), level
+
+
 def test_non_contiguous_input_is_handled():
     q, u, vt, x = synthetic_layer(128, 512, 2, 4, seed=4, device=dev())
     wide = torch.randn(4, 1024, device=dev()).half()
