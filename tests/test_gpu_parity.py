@@ -279,6 +279,31 @@ def test_full_size_properties_largest_decode_shape():
     assert_close(y[:, rows].cpu().numpy(), exact, "spot rows vs fp64", 1e-2, 2e-3)
 
 
+@pytest.mark.parametrize("M,N", [(28672, 8192), (8192, 28672), (8192, 8192), (1024, 8192)])
+def test_llama_70b_shapes_spot_rows_on_every_path(M, N):
+    """The four linear shapes of the 70B configuration with 3 blocks, at 1, 4, 8 and 64 tokens (decode
+    kernel, strip kernel, rebuild + dense kernel): sampled rows against the float64 closed form, and the
+    paths against one another over all rows."""
+    I = 3
+    q, u, vt, x = synthetic_layer(M, N, I, 64, seed=31, device=dev())
+    rows = [0, 1, 63, 64, M // 2 + 5, M - 2, M - 1]
+    exact = O.forward_exact(np.stack([qq.cpu().numpy().reshape(M, N // 8)[rows].reshape(-1) for qq in q]),
+                            u[:, rows].cpu().numpy(), vt.cpu().numpy(), x.cpu().numpy())
+    f = IU.bitstack_forward_hip
+    plans = {T: _lib.decode_plan(I, M, N, 16, T)[0] for T in (1, 4, 8, 64)}
+    assert plans[1] > 0 and plans[4] > 0 and plans[8] == 0 and plans[64] == 0      # decode kernel up to 4 tokens only
+    ys = {}
+    for T in (1, 4, 8, 64):
+        print(f"70B shape M={M} N={N} I={I} T={T}", flush=True)
+        y = f(q, u, vt, x[:T].contiguous())
+        assert tuple(y.shape) == (T, M)
+        assert_close(y[:, rows].cpu().numpy(), exact[:T], f"T={T} spot rows vs fp64", 1e-2, 2e-3)
+        ys[T] = y.float()
+    scale = float(ys[64].abs().max())
+    for T in (1, 4, 8):
+        assert float((ys[T] - ys[64][:T]).abs().max()) <= 4e-3 * scale, T
+
+
 # ------------------------------------------------------------ module levels
 def build_module(M, N, I, bias, seed):
     q, u, vt, x = synthetic_layer(M, N, I, 3, seed=seed, signed_factors=True)
