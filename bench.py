@@ -326,6 +326,22 @@ def main():
             tp = sum(perp) * 1e-3
             pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
                             "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+            if T >= 512:
+                # beside it, the module's level 3 on the same layers: this library's rebuild kernel, then
+                # torch's F.linear (hipBLASLt) as in the reference's levels 2-4; never the headline
+                import torch.nn.functional as F
+                from bitstack_amd.utils.inference_utils import unpack_and_reconstruct_w_hip
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t3 = 0.0
+                for L in lp:
+                    for r in range(4):
+                        if r == 1:
+                            e0.record()
+                        F.linear(L.x, unpack_and_reconstruct_w_hip(L.q, L.u, L.vt))
+                    e1.record()
+                    torch.cuda.synchronize()
+                    t3 += e0.elapsed_time(e1) / 3 * 1e-3
+                pre[f"T{T}"]["level3_rebuild_plus_torch_linear_useful_tflops"] = round(useful / t3 / 1e12, 1)
             detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
                         "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
                        for L, ms in zip(lp, perp)]
