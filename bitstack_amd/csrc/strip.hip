@@ -46,8 +46,8 @@ struct StripGroup {
     float *ssq;     // [strip groups of matrix 0][T]: sum of x^2 over the group's columns (for an RMS scale), or null
 };
 
-template <int TT>
-__global__ __launch_bounds__(256, 4) void strip_forward_kernel(
+template <int TT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
     const StripGroup grp, const half_t *__restrict__ x, int N, int K, int T) {
     extern __shared__ __attribute__((aligned(16))) half_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -93,13 +93,15 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
     const int64_t row_bytes = N >> 3;
     const int64_t block_bytes = (int64_t)M * row_bytes;
 
-    const int sr = tid & 15, sp = tid >> 4;         // staging role: rank, piece of 8 columns
+    const int sr = tid & 15, sp = (tid >> 4) & 15;  // staging role: rank, piece of 8 columns
+    const int spair = tid >> 8;                     // ... and which of the WAVES / 4 pairs staged side by side
     const int sh_byte = 24 - 8 * g;                 // brings the lane's byte of a sign word to the top
     const int acol = 8 * (lm >> 2) + (lm & 3);
     const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
 
     const int first_row = row_begin + wave * 16;
-    const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
+    constexpr int NT = 64 * WAVES, RS = 16 * WAVES;  // threads, rows per step of the workgroup
+    const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / RS) * RS;
     // Addresses are a wave-uniform 64-bit base (block, strip: scalar arithmetic) plus a 32-bit
     // offset per lane that depends on the row only and is renewed once per row step; worked out
     // per request in 64 bits per lane, the multiplications were a fifth of the kernel's VALU time.
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
             pf_i = 0;
             if (++pf_q == ns) {
                 pf_q = 0;
-                pf_m0 += 64;
+                pf_m0 += RS;
                 set_row(pf_m0);
             }
         }
@@ -144,26 +146,27 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
     request(b_n1, sw_n1);
 
     // x image: token rows beyond T are zero
-    for (int idx = tid; idx < TT * 16 * ns * 16; idx += 256) {
+    for (int idx = tid; idx < TT * 16 * ns * 16; idx += NT) {
         const int t = idx / (ns * 16), piece = idx % (ns * 16);
         half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (t < T) v = *reinterpret_cast<const half8_t *>(x + (int64_t)t * N + n0 + 8 * piece);
         *reinterpret_cast<half8_t *>(xl + t * xstride + 8 * piece) = v;
     }
     // vt slices, four (strip, block) pairs at a time so that their loads are in flight together
-    for (int q0 = 0; q0 < ns * I; q0 += 4) {
+    constexpr int SIDE = WAVES / 4;                 // 256 threads stage one (strip, block) pair
+    for (int q0 = 0; q0 < ns * I; q0 += 4 * SIDE) {
         half8_t v[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const int qi = min(q0 + k, ns * I - 1), q = qi / I, i = qi - q * I;
+            const int qi = min(q0 + k * SIDE + spair, ns * I - 1), q = qi / I, i = qi - q * I;
             v[k] = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
             if (sr < K) v[k] = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + q * SF_COLS + 8 * sp);
         }
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            if (q0 + k < ns * I) {
+            if (q0 + k * SIDE + spair < ns * I) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) vl[(q0 + k) * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[k][e];
+                for (int e = 0; e < 8; e++) vl[(q0 + k * SIDE + spair) * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[k][e];
             }
         }
     }
@@ -171,25 +174,29 @@ __global__ __launch_bounds__(256, 4) void strip_forward_kernel(
 
     // sum of squares of every token over this group's columns, once per strip group
     if (grp.ssq && first_matrix && row_begin == 0) {
-        const int t = tid >> 3, sub = tid & 7;
-        float q = 0.f;
-        if (t < TT * 16) {
-            for (int c = sub * 8; c < ns * SF_COLS; c += 64) {
-                const half8_t v = *reinterpret_cast<const half8_t *>(xl + t * xstride + c);
+        const int sub = tid & 7;
+        // eight lanes per token row, NT / 8 rows per pass (48 token rows need two passes of 256 threads)
+        for (int t0 = 0; t0 < TT * 16; t0 += NT / 8) {
+            const int t = t0 + (tid >> 3);
+            float q = 0.f;
+            if (t < TT * 16) {
+                for (int c = sub * 8; c < ns * SF_COLS; c += 64) {
+                    const half8_t v = *reinterpret_cast<const half8_t *>(xl + t * xstride + c);
 #pragma unroll
-                for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+                    for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+                }
             }
+            q += __shfl_xor(q, 1, 64);
+            q += __shfl_xor(q, 2, 64);
+            q += __shfl_xor(q, 4, 64);
+            if (sub == 0 && t < T) grp.ssq[group * T + t] = q;
         }
-        q += __shfl_xor(q, 1, 64);
-        q += __shfl_xor(q, 2, 64);
-        q += __shfl_xor(q, 4, 64);
-        if (sub == 0 && t < T) grp.ssq[group * T + t] = q;
     }
 
     // this lane's x fragments: token lm of a tile, columns 32 (s / 2) + 8 g + 4 (s % 2) .. + 3 of patch s
     const half_t *xfrag = xl + lm * xstride + 8 * g;
 
-    for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += 64) {
+    for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += RS) {
         float4_t yacc[TT];
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
@@ -262,42 +269,60 @@ size_t strip_lds(int I, int tt, int sg) {
     return ((size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
 }
 
-// Strips per workgroup: as many (a power of two up to 8) as keep three workgroups on a
-// CU and a grid of at least one workgroup per CU; then as
-// many row groups as fill the resident slots once.
+// Workgroups of 8 waves (two per CU): they share one vt image, so a CU holds 16 waves with half the
+// LDS four-wave workgroups would need (at 16 blocks two of those, 8 waves, were all a CU could hold).
+constexpr int STRIP_WAVES = 8;
+
+// Strips per workgroup (a power of two up to 8) and row groups: of the choices that keep two
+// workgroups on a CU and give every CU one, the one with the least work on the busiest CU -
+// workgroups per CU x row steps per workgroup x strips per workgroup, which is what the rounding of
+// rows to whole steps of 128 and of workgroups to whole CUs changes - and among equals the most
+// strips (fewest partial sums).
 StripPlan make_strip_plan(int I, int M, int N, int T) {
-    StripPlan p;
-    p.tt = token_tiles(T);
-    const int strips = N / SF_COLS, cap = 4, want = 3;
-    p.sg = 1;
-    for (int sg = 8; sg > 1; sg >>= 1) {
-        if (strip_lds(I, p.tt, sg) * want > 160 * 1024) continue;
-        if (bs_cdiv(strips, sg) * bs_cdiv(M, 64) < 256) continue;
+    StripPlan best;
+    best.sg = 0;
+    long best_cost = 0;
+    const int tt = token_tiles(T), rs = 16 * STRIP_WAVES, cap = 16 / STRIP_WAVES;
+    const int strips = N / SF_COLS;
+    for (int sg = 8; sg >= 1; sg >>= 1) {
+        StripPlan p;
+        p.tt = tt;
         p.sg = sg;
-        break;
+        p.lds = strip_lds(I, tt, sg);
+        if (sg > 1 && p.lds * cap > 160 * 1024) continue;
+        if (sg > 1 && bs_cdiv(strips, sg) * bs_cdiv(M, rs) < 256) continue;
+        int per_cu = (int)((160 * 1024) / p.lds);
+        if (per_cu > cap) per_cu = cap;
+        if (per_cu < 1) per_cu = 1;
+        p.groups = (int)bs_cdiv(strips, sg);
+        const int per_line = 8 / sg;
+        p.gx = (int)bs_cdiv(p.groups, per_line) * per_line;
+        int row_groups = (256 * per_cu) / p.gx;
+        if (row_groups < 1) row_groups = 1;
+        p.rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), rs) * rs;
+        p.row_groups = (int)bs_cdiv(M, p.rows_per_wg);
+        const long cost = (long)bs_cdiv(p.gx * p.row_groups, 256) * (p.rows_per_wg / rs) * sg;
+        if (best.sg == 0 || cost < best_cost) {
+            best = p;
+            best_cost = cost;
+        }
     }
-    p.lds = strip_lds(I, p.tt, p.sg);
-    int per_cu = (int)((160 * 1024) / p.lds);
-    if (per_cu > cap) per_cu = cap;
-    if (per_cu < 1) per_cu = 1;
-    p.groups = (int)bs_cdiv(strips, p.sg);
-    const int per_line = 8 / p.sg;
-    p.gx = (int)bs_cdiv(p.groups, per_line) * per_line;
-    int row_groups = (256 * per_cu) / p.gx;
-    if (row_groups < 1) row_groups = 1;
-    p.rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
-    p.row_groups = (int)bs_cdiv(M, p.rows_per_wg);
-    return p;
+    return best;
+}
+
+template <int TT, int WAVES>
+int launch_ttw(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
+    static size_t granted[BS_MAX_DEVICES] = {};
+    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT, WAVES>, lds, granted);
+    if (st != BS_OK) return st;
+    strip_forward_kernel<TT, WAVES><<<grid, 64 * WAVES, lds, s>>>(grp, x, N, K, T);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
 }
 
 template <int TT>
 int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
-    static size_t granted[BS_MAX_DEVICES] = {};
-    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT>, lds, granted);
-    if (st != BS_OK) return st;
-    strip_forward_kernel<TT><<<grid, 256, lds, s>>>(grp, x, N, K, T);
-    BS_LAUNCH_CHECK();
-    return BS_OK;
+    return launch_ttw<TT, STRIP_WAVES>(grp, grid, lds, x, N, K, T, s);
 }
 
 }  // namespace

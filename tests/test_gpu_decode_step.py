@@ -344,6 +344,9 @@ def test_decoder_round_trips_through_a_checkpoint(tmp_path):
                                               ([(2, 1024), (3, 1024)], 2048, 1, "swiglu"),
                                               ([(2, 256), (1, 256)], 512, 5, "swiglu"),
                                               ([(2, 512), (3, 128)], 1024, 20, "none"),
+                                              # three token tiles: more token rows than one pass of the sum of squares takes
+                                              ([(2, 512), (3, 128)], 1024, 40, "none"),
+                                              ([(2, 256), (2, 256)], 512, 48, "swiglu"),
                                               ([(2, 300)], 1536, 3, "none")])
 def test_group_forward_with_input_rms(shapes, N, T, mode):
     """bs_forward_group_rms: the RMSNorm in front of the matrices without a launch of its own.  The

@@ -330,9 +330,12 @@ def test_full_size_properties_strip_kernel():
     # and a 40-token call (three token tiles) repeats them
     x40 = torch.cat([x, x, x[:8]])
     y40 = f(q, u, vt, x40)
-    assert torch.equal(y40[:16], y) and torch.equal(y40[16:32], y) and torch.equal(y40[32:], y[:8])
     yf = y.float()
     scale = float(yf.abs().max())
+    # (three token tiles leave room for fewer strips per workgroup, so the strips' partial sums are
+    # added in other groups: the same numbers up to the fp32 summation order)
+    assert torch.equal(y40[:16], y40[16:32]) and torch.equal(y40[32:], y40[:8])
+    assert float((y40[:16].float() - yf).abs().max()) <= 1e-3 * scale
     assert float((f(q, u, vt, x * 2).float() - 2 * yf).abs().max()) <= 2e-3 * scale           # linearity in x
     parts = f(q[:4], u[:4], vt[:4], x).float() + f(q[4:], u[4:], vt[4:], x).float()
     assert float((parts - yf).abs().max()) <= 4e-3 * scale                                    # block additivity (w is rounded per call)
