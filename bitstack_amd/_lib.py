@@ -13,8 +13,7 @@ import threading
 import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-# BITSTACK_AMD_LIB points at another build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("BITSTACK_AMD_LIB") or os.path.join(_CSRC, "libbitstack_hip.so")
+LIB_PATH = os.path.join(_CSRC, "libbitstack_hip.so")
 
 # name -> (restype, argtypes); mirrors include/bitstack_hip.h one to one
 _P, _I, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
@@ -29,6 +28,7 @@ SIGNATURES = {
     "bs_decode_plan": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P]),
     "bs_forward": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _L, _P]),
     "bs_linear_f16": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
+    "bs_linear_plan": (_I, [_I, _I, _I, _P, _P, _P, _P]),
 }
 
 
@@ -83,6 +83,13 @@ def decode_plan(I, M, N, K, T):
     return tuple(v.value for v in vals)
 
 
+def linear_plan(T, M, N):
+    """(tile_tokens, tile_features, k_step, k_tail) of the dense kernel for these dimensions."""
+    vals = [ctypes.c_int(0) for _ in range(4)]
+    check(lib().bs_linear_plan(T, M, N, *[ctypes.byref(v) for v in vals]), "bs_linear_plan")
+    return tuple(v.value for v in vals)
+
+
 def error_string(status: int) -> str:
     return lib().bs_error_string(int(status)).decode()
 
@@ -116,14 +123,26 @@ def stream_ptr(dev):
 
 
 _workspaces: dict = {}
+_retired: list = []
 
 
 def workspace(dev, nbytes: int):
     """Per-(device, stream) scratch tensor, grown on demand.  Kernels on one
-    stream are ordered, so reusing it across calls on that stream is safe."""
+    stream are ordered, so reusing it across calls on that stream is safe.
+
+    A buffer that is outgrown is kept alive for the life of the process, never
+    handed back to the allocator: a HIP graph captured while it was current has
+    its address baked in, and its replays must keep writing into memory nobody
+    else owns.  (A graph captured before a growth still uses the old buffer; it
+    stays correct, it just does not share scratch with later eager calls.)"""
     key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
-    buf = _workspaces.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _workspaces[key] = buf
+    with _lock:
+        buf = _workspaces.get(key)
+        if buf is None or buf.numel() < nbytes:
+            if buf is not None:
+                _retired.append(buf)
+            # grow geometrically so that a sequence of slowly growing requests retires few buffers
+            size = max(nbytes, 1 << 20, 0 if buf is None else 2 * buf.numel())
+            buf = torch.empty(size, dtype=torch.uint8, device=dev)
+            _workspaces[key] = buf
     return buf

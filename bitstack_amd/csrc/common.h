@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/bitstack_hip.h"
 
 #define BS_VERSION_NUMBER 100  // 0.1.0
@@ -27,15 +29,21 @@ static inline int64_t bs_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Kernels that need more than 64 KB of dynamic LDS must be allowed to, once per kernel AND
 // per device (the attribute lives with the device's copy of the code).  `granted[d]` is the
 // size already allowed on device d; the caller keeps one such array per kernel.
+// Host threads may race here: the table entries are atomics (a torn read could skip a grant
+// that was never made), and setting the attribute twice to the same or a larger size is harmless.
 constexpr int BS_MAX_DEVICES = 64;
-static inline int bs_allow_lds(const void *kernel, size_t bytes, size_t *granted) {
+typedef std::atomic<size_t> bs_lds_grant;
+static inline int bs_allow_lds(const void *kernel, size_t bytes, bs_lds_grant *granted) {
     if (bytes <= 64 * 1024) return BS_OK;
     int dev = 0;
     BS_HIP_TRY(hipGetDevice(&dev));
     const bool tracked = dev >= 0 && dev < BS_MAX_DEVICES;
-    if (tracked && granted[dev] >= bytes) return BS_OK;
+    if (tracked && granted[dev].load(std::memory_order_acquire) >= bytes) return BS_OK;
     BS_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
-    if (tracked) granted[dev] = bytes;
+    if (tracked) {
+        size_t seen = granted[dev].load(std::memory_order_relaxed);
+        while (seen < bytes && !granted[dev].compare_exchange_weak(seen, bytes, std::memory_order_release)) {}
+    }
     return BS_OK;
 }
 

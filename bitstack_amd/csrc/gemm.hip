@@ -322,7 +322,7 @@ int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y
                  hipStream_t s) {
     constexpr int BT = WT * AT * 32, BF = WF * AF * 32;
     constexpr size_t lds = (size_t)2 * (BT + BF) * lds_stride(GK) * sizeof(half_t);
-    static size_t granted[2][BS_MAX_DEVICES] = {};
+    static bs_lds_grant granted[2][BS_MAX_DEVICES];
     int st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>, lds, granted[0]);
     if (st == BS_OK) st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>, lds, granted[1]);
     if (st != BS_OK) return st;
@@ -336,32 +336,59 @@ int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y
 
 }  // namespace
 
+// Which kernel a dense forward of these dimensions runs: tokens x features per workgroup
+// (0 x 0 for the one-wave-per-output kernel), and whether the contracted range ends in a
+// partial k-step.
+struct LinearTile { int bt, bf, gk; };
+static LinearTile linear_tile(int T, int M, int N, bool aligned) {
+    if (!(N % 8 == 0 && aligned)) return {0, 0, 0};
+    if (T <= 32 && N % 16 == 0) return {32, 32, 0};                       // linear_skinny_kernel
+    if (T <= 128) return M >= 8192 ? LinearTile{128, 64, 64} : LinearTile{128, 32, 128};
+    // The largest tile whose grid still covers most of the 256 CUs: 256 x 256 and
+    // 128 x 256 (8 waves) move the fewest bytes per flop; 128 x 128 and 64 x 64
+    // (4 waves, two workgroups per CU) keep a small problem spread over the chip.
+    const auto wgs = [&](int bt, int bf) { return bs_cdiv(T, bt) * bs_cdiv(M, bf); };
+    return wgs(256, 256) >= 160 ? LinearTile{256, 256, 32} :
+           wgs(128, 256) >= 160 ? LinearTile{128, 256, 64} :
+           wgs(128, 128) >= 192 ? LinearTile{128, 128, 64} : LinearTile{64, 64, 128};
+}
+
 int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, half_t *y,
                          int T, int M, int N, hipStream_t s) {
-    if (N % 8 == 0 && bs_aligned(x, 16) && bs_aligned(w, 16)) {
-        int st = BS_OK;
-        if (T <= 32 && N % 16 == 0) {
-            linear_skinny_kernel<1, 8, 8><<<(int)bs_cdiv(M, 32), 512, 0, s>>>(x, w, bias, y, T, M, N);
-        } else if (T <= 128) {
-            st = M >= 8192 ? launch_tiled<2, 2, 2, 1, 64>(x, w, bias, y, T, M, N, s)
-                           : launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
-        } else {
-            // The largest tile whose grid still covers most of the 256 CUs: 256 x 256 and
-            // 128 x 256 (8 waves) move the fewest bytes per flop; 128 x 128 and 64 x 64
-            // (4 waves, two workgroups per CU) keep a small problem spread over the chip.
-            const auto wgs = [&](int bt, int bf) { return bs_cdiv(T, bt) * bs_cdiv(M, bf); };
-            st = wgs(256, 256) >= 160 ? launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s) :
-                 wgs(128, 256) >= 160 ? launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s) :
-                 wgs(128, 128) >= 192 ? launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s)
-                                      : launch_tiled<2, 2, 1, 1, 128>(x, w, bias, y, T, M, N, s);
-        }
-        if (st != BS_OK) return st;
-    } else {
+    const LinearTile tile = linear_tile(T, M, N, bs_aligned(x, 16) && bs_aligned(w, 16));
+    int st = BS_OK;
+    if (tile.bt == 0) {
         int64_t blocks = bs_cdiv((int64_t)T * M, 4);
         if (blocks > 256 * 64) blocks = 256 * 64;
         linear_generic_kernel<<<(int)blocks, 256, 0, s>>>(x, w, bias, y, T, M, N);
+    } else if (tile.gk == 0) {
+        linear_skinny_kernel<1, 8, 8><<<(int)bs_cdiv(M, 32), 512, 0, s>>>(x, w, bias, y, T, M, N);
+    } else if (tile.bt == 128 && tile.bf == 64) {
+        st = launch_tiled<2, 2, 2, 1, 64>(x, w, bias, y, T, M, N, s);
+    } else if (tile.bt == 128 && tile.bf == 32) {
+        st = launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
+    } else if (tile.bt == 256) {
+        st = launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s);
+    } else if (tile.bf == 256) {
+        st = launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+    } else if (tile.bf == 128) {
+        st = launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+    } else {
+        st = launch_tiled<2, 2, 1, 1, 128>(x, w, bias, y, T, M, N, s);
     }
+    if (st != BS_OK) return st;
     BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
+extern "C" int bs_linear_plan(int T, int M, int N, int *tile_tokens, int *tile_features, int *k_step, int *k_tail) {
+    if (!tile_tokens || !tile_features || !k_step || !k_tail) return BS_ERR_NULL;
+    if (T <= 0 || M <= 0 || N <= 0) return BS_ERR_SHAPE;
+    const LinearTile t = linear_tile(T, M, N, true);
+    *tile_tokens = t.bt;
+    *tile_features = t.bf;
+    *k_step = t.gk;
+    *k_tail = t.gk > 0 && N % t.gk != 0;
     return BS_OK;
 }
 

@@ -730,7 +730,7 @@ struct GroupArgs {          // host-side view of one call
 template <int T, int WAVES, int R>
 int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
     const size_t lds = (size_t)2 * T * 16384 + (size_t)2 * WAVES * T * 64;
-    static size_t granted[BS_MAX_DEVICES] = {};      // per instantiation
+    static bs_lds_grant granted[BS_MAX_DEVICES];      // per instantiation
     const int st = bs_allow_lds((const void *)gemv_kernel<T, WAVES, R>, lds, granted);
     if (st != BS_OK) return st;
     gemv_kernel<T, WAVES, R><<<p.grid, 64 * WAVES, lds, s>>>(grp, x, N, K, p.n_chunks);
@@ -738,21 +738,27 @@ int launch_one(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int 
     return BS_OK;
 }
 
+// Only the (WAVES, R) pairs make_plan can choose for T tokens exist; any other pair is refused
+// rather than run on a tile of another height (the reduce kernel and the partial layout are
+// built for exactly waves * R * 16 rows per tile).
 template <int T>
 int launch_T(const Plan &p, const GemvGroup &grp, const half_t *x, int N, int K, hipStream_t s) {
-    if (p.waves == 16) {
-        if constexpr (T == 1) return launch_one<T, 16, 4>(p, grp, x, N, K, s);
-        else return BS_ERR_SHAPE;
+    const int w = p.waves, r = p.R;
+    if constexpr (T == 1) {
+        if (w == 16 && r == 4) return launch_one<1, 16, 4>(p, grp, x, N, K, s);
+        if (w == 8 && r == 4) return launch_one<1, 8, 4>(p, grp, x, N, K, s);
+    } else if constexpr (T == 2) {
+        if (w == 8 && r == 2) return launch_one<2, 8, 2>(p, grp, x, N, K, s);
+    } else {
+        if (w == 8 && r == 4) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
+        if (w == 8 && r == 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
     }
-    if (p.waves == 8) {
-        if constexpr (T == 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
-        else if (p.R == 4) return launch_one<T, 8, 4>(p, grp, x, N, K, s);
-        else if constexpr (T > 2) return launch_one<T, 8, 2>(p, grp, x, N, K, s);
-        else return BS_ERR_SHAPE;
+    if constexpr (T <= 2) {
+        if (w == 4 && r == 4) return launch_one<T, 4, 4>(p, grp, x, N, K, s);
     }
-    if (p.R == 4) return launch_one<T, 4, 4>(p, grp, x, N, K, s);
-    if (p.R == 2) return launch_one<T, 4, 2>(p, grp, x, N, K, s);
-    return launch_one<T, 4, 1>(p, grp, x, N, K, s);
+    if (w == 4 && r == 2) return launch_one<T, 4, 2>(p, grp, x, N, K, s);
+    if (w == 4 && r == 1) return launch_one<T, 4, 1>(p, grp, x, N, K, s);
+    return BS_ERR_SHAPE;
 }
 
 bool gemv_shape_ok(int I, int M, int N, int T) {
@@ -861,32 +867,35 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         if (a.n != 2 || a.M[0] != a.M[1]) return BS_ERR_SHAPE;
         ldy = a.M[0];
     }
+    // Tokens go in passes of tp, the last one possibly shorter.  Every pass length has its own
+    // plan (instantiation, grid, partial layout): the kernel a plan names exists for that token
+    // count only.  Passes run one after the other on the stream and share the workspace.
     const int tp = pass_tokens(T);
-    const Plan p = make_plan(a.I, a.M, a.n, N, tp);
-    if (!workspace || workspace_bytes < p.part_total * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
     float *part = (float *)workspace;
-    GemvGroup g;
-    RedGroup r;
-    g.n = r.n = a.n;
-    r.mode = mode;
-    r.xin = nullptr;
-    r.n_in = N;
-    r.eps = eps;
-    r.ssq = nullptr;
-    r.ssq_n = 0;
-    int y_off = 0, blocks = 0;
-    for (int j = 0; j < a.n; j++) {
-        g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
-                         p.first_wg[j], p.sp[j], p.pair};
-        r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks, p.sp[j],
-                        p.pair};
-        y_off += a.M[j];
-        if (mode != EPI_SWIGLU || j == 0) blocks += tp * (int)bs_cdiv(a.M[j], RED_OUT);
-    }
-    for (int j = a.n; j < GEMV_MAX_GROUP; j++) { g.m[j] = g.m[0]; r.m[j] = r.m[0]; }
     for (int t0 = 0; t0 < T; t0 += tp) {
         const int tn = (T - t0 < tp) ? T - t0 : tp;
+        const Plan p = make_plan(a.I, a.M, a.n, N, tn);
+        if (!workspace || workspace_bytes < p.part_total * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
+        GemvGroup g;
+        RedGroup r;
+        g.n = r.n = a.n;
+        r.mode = mode;
+        r.n_in = N;
+        r.eps = eps;
+        r.ssq = nullptr;
+        r.ssq_n = 0;
+        int y_off = 0, blocks = 0;
+        for (int j = 0; j < a.n; j++) {
+            g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
+                             p.first_wg[j], p.sp[j], p.pair};
+            r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks,
+                            p.sp[j], p.pair};
+            y_off += a.M[j];
+            if (mode != EPI_SWIGLU || j == 0) blocks += tn * (int)bs_cdiv(a.M[j], RED_OUT);
+        }
+        for (int j = a.n; j < GEMV_MAX_GROUP; j++) { g.m[j] = g.m[0]; r.m[j] = r.m[0]; }
         const half_t *xp = x + (int64_t)t0 * N;
+        r.xin = input_rms ? xp : nullptr;
         int st;
         switch (tn) {
             case 1: st = launch_T<1>(p, g, xp, N, K, s); break;
@@ -895,23 +904,23 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
             default: st = launch_T<4>(p, g, xp, N, K, s); break;
         }
         if (st != BS_OK) return st;
-        // the partial areas are laid out for tp tokens; a shorter last pass uses its own stride
-        RedGroup rr = r;
-        if (input_rms) rr.xin = xp;
-        int nblocks = blocks;
-        if (tn != tp) {
-            nblocks = 0;
-            for (int j = 0; j < a.n; j++) {
-                rr.m[j].first_block = nblocks;
-                if (mode != EPI_SWIGLU || j == 0) nblocks += tn * (int)bs_cdiv(a.M[j], RED_OUT);
-            }
-        }
-        gemv_reduce_kernel<1><<<nblocks, RED_OUT * RED_SL, 0, s>>>(rr, residual ? residual + (int64_t)t0 * ldy : nullptr,
-                                                                y + (int64_t)t0 * ldy, tn, ldy,
-                                                                p.waves * p.R * 16, p.n_chunks);
+        gemv_reduce_kernel<1><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual ? residual + (int64_t)t0 * ldy : nullptr,
+                                                               y + (int64_t)t0 * ldy, tn, ldy,
+                                                               p.waves * p.R * 16, p.n_chunks);
         BS_LAUNCH_CHECK();
     }
     return BS_OK;
+}
+
+// Scratch the factor-through path needs: the largest partial area over its passes.
+int64_t gemv_part_floats(const int *I, const int *M, int n, int N, int T) {
+    const int tp = pass_tokens(T), tail = T % tp;
+    int64_t need = make_plan(I, M, n, N, tp).part_total;
+    if (tail) {
+        const int64_t t2 = make_plan(I, M, n, N, tail).part_total;
+        if (t2 > need) need = t2;
+    }
+    return need;
 }
 
 }  // namespace
@@ -926,8 +935,7 @@ int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, 
     const int path = group_path(I, M, n, N, K, T);
     if (path < 0) return 0;
     if (path == 1) return strip_part_floats(I, M, n, N, K, T) * (int64_t)sizeof(float);
-    const Plan p = make_plan(I, M, n, N, pass_tokens(T));
-    return p.part_total * (int64_t)sizeof(float);
+    return gemv_part_floats(I, M, n, N, T) * (int64_t)sizeof(float);
 }
 
 // Which instantiation and grid a decode forward of these dimensions runs

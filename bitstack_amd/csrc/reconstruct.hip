@@ -241,7 +241,7 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
         int rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
         row_groups = (int)bs_cdiv(M, rows_per_wg);
         const size_t lds = lds_need;
-        static size_t granted[BS_MAX_DEVICES] = {};
+        static bs_lds_grant granted[BS_MAX_DEVICES];
         const int st = bs_allow_lds((const void *)reconstruct_tile_kernel<PACKED>, lds, granted);
         if (st != BS_OK) return st;
         dim3 grid((unsigned)bs_cdiv(strips, 8) * 8, row_groups);

@@ -312,7 +312,7 @@ StripPlan make_strip_plan(int I, int M, int N, int T) {
 
 template <int TT, int WAVES>
 int launch_ttw(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
-    static size_t granted[BS_MAX_DEVICES] = {};
+    static bs_lds_grant granted[BS_MAX_DEVICES];
     const int st = bs_allow_lds((const void *)strip_forward_kernel<TT, WAVES>, lds, granted);
     if (st != BS_OK) return st;
     strip_forward_kernel<TT, WAVES><<<grid, 64 * WAVES, lds, s>>>(grp, x, N, K, T);

@@ -40,6 +40,8 @@ class LlamaShape:
     rope_theta: float = 500000.0
     rms_eps: float = 1e-5
     k: int = 16
+    # Hugging Face `rope_scaling` / `rope_parameters` dictionary (None: plain RoPE); see rope_inv_freq
+    rope_scaling: dict | None = None
 
     @property
     def head_dim(self):
@@ -58,6 +60,33 @@ class LlamaShape:
 
     def dense_bytes(self):
         return 2 * 2 * self.vocab * self.hidden            # embed_tokens + lm_head, fp16
+
+
+def rope_inv_freq(head_dim: int, theta: float, scaling: dict | None = None) -> torch.Tensor:
+    """Inverse RoPE frequencies [head_dim / 2] (float32, CPU) for a Hugging Face rope configuration.
+
+    None / "default": theta^(-2j/d).  "linear": those divided by `factor`.  "llama3" (the released
+    Llama-3.1 / 3.2 checkpoints the reference evaluates): wavelengths above
+    original_max_position_embeddings / low_freq_factor are divided by `factor`, those below
+    original / high_freq_factor are kept, and the band between is blended linearly in
+    original / wavelength.  Any other type raises: the tables would silently be wrong."""
+    import math
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    kind = (scaling or {}).get("rope_type", (scaling or {}).get("type", "default")) or "default"
+    if kind == "default":
+        return inv
+    if kind == "linear":
+        return inv / float(scaling["factor"])
+    if kind != "llama3":
+        raise ValueError(f"rope scaling type {kind!r} is not supported (default, linear, llama3 are)")
+    factor, lo_f, hi_f = float(scaling["factor"]), float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
+    old_len = float(scaling["original_max_position_embeddings"])
+    wavelen = 2 * math.pi / inv
+    smooth = (old_len / wavelen - lo_f) / (hi_f - lo_f)
+    blended = (1 - smooth) * inv / factor + smooth * inv
+    out = torch.where(wavelen > old_len / lo_f, inv / factor, inv)
+    mid = (wavelen <= old_len / lo_f) & (wavelen >= old_len / hi_f)
+    return torch.where(mid, blended, out)
 
 
 LLAMA_8B = LlamaShape()
@@ -134,7 +163,7 @@ class SyntheticLlamaDecoder:
         d = shape.head_dim
         self.kcache = torch.zeros(shape.layers, batch, shape.kv_heads, max_len, d, device=self.dev, dtype=torch.float16)
         self.vcache = torch.zeros_like(self.kcache)
-        inv = 1.0 / (shape.rope_theta ** (torch.arange(0, d, 2, device=self.dev, dtype=torch.float32) / d))
+        inv = rope_inv_freq(d, shape.rope_theta, shape.rope_scaling).to(self.dev)
         ang = torch.arange(max_len, device=self.dev, dtype=torch.float32)[:, None] * inv[None, :]
         self.cos, self.sin = ang.cos().half().contiguous(), ang.sin().half().contiguous()   # [max_len, d/2]
         self.pos = torch.zeros(1, device=self.dev, dtype=torch.long)       # next position to write
@@ -155,8 +184,11 @@ class SyntheticLlamaDecoder:
         from bitstack_amd.utils import checkpoint as ck
         with open(os.path.join(path, "config.json"), "r") as f:
             hf = json.load(f)
-        rope = hf.get("rope_theta") or (hf.get("rope_parameters") or {}).get("rope_theta", 10000.0)
-        shape = LlamaShape(layers=hf["num_hidden_layers"], hidden=hf["hidden_size"], intermediate=hf["intermediate_size"],
+        rope_par = hf.get("rope_parameters") or {}
+        rope = hf.get("rope_theta") or rope_par.get("rope_theta", 10000.0)
+        scaling = hf.get("rope_scaling") or (rope_par if rope_par.get("rope_type", "default") != "default" else None)
+        rope_inv_freq(2, float(rope), scaling)              # raises here, before any weight is read, if unsupported
+        shape = LlamaShape(rope_scaling=scaling, layers=hf["num_hidden_layers"], hidden=hf["hidden_size"], intermediate=hf["intermediate_size"],
                            heads=hf["num_attention_heads"], kv_heads=hf.get("num_key_value_heads", hf["num_attention_heads"]),
                            vocab=hf["vocab_size"], rope_theta=float(rope), rms_eps=float(hf.get("rms_norm_eps", 1e-5)))
         if hf.get("head_dim", shape.head_dim) != shape.head_dim:

@@ -130,6 +130,17 @@ int bs_linear_f16(const void *x, const void *w, const void *bias, void *y,
                   int T, int M, int N, void *stream);
 
 /*
+ * Introspection for benchmarks and tests: the workgroup tile (tokens x output
+ * features), the k-step and whether the last k-step is partial (N not a multiple
+ * of the step) of the dense kernel bs_linear_f16 - and bs_forward above 48
+ * tokens - runs for these dimensions with 16-byte aligned buffers.  32 x 32
+ * with *k_step == 0 is the no-LDS kernel for up to 32 tokens, 0 x 0 the
+ * one-wave-per-output kernel (N % 8 != 0).  No counterpart in the reference
+ * (F.linear picks a vendor kernel).
+ */
+int bs_linear_plan(int T, int M, int N, int *tile_tokens, int *tile_features, int *k_step, int *k_tail);
+
+/*
  * ---- decode step: several matrices per launch, fused epilogues -----------
  * One decode forward (T <= 48 tokens; more than 8 need N % 128 == 0) of up to 4 compressed matrices that read
  * the same x, in one kernel pair: what q_proj/k_proj/v_proj (or gate_proj/

@@ -173,6 +173,28 @@ def test_forward_decode_matches_oracle(I, M, N, T):
         assert_close(y, l0, "vs level-0 order")
 
 
+@pytest.mark.parametrize("I,M,N,T", [(40, 1024, 4096, 5), (40, 4096, 4096, 5), (40, 4096, 4096, 7), (40, 1024, 4096, 6)])
+def test_forward_decode_two_passes_of_unequal_length(I, M, N, T):
+    """Stacks too long for the strip kernel (its vt image would not fit in LDS) take the decode kernel
+    in two passes (3 + 2, 3 + 3, 4 + 3 tokens); the shorter pass has a plan of its own, and every row of
+    every token must come out (a tail pass run on the first pass's tile height left half of each row
+    tile unwritten)."""
+    print(f"forward two passes I={I} M={M} N={N} T={T}", flush=True)
+    assert _lib.decode_plan(I, M, N, 16, T)[0] > 0         # the decode kernel, not the strip kernel
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=I + T)
+    exact = C.forward_f64(q.numpy(), u.numpy(), vt.numpy(), x.numpy())
+    qd, ud, vd, xd = q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())
+    # poison the scratch the call will use, so an unwritten partial cannot pass by luck
+    ws = _lib.workspace(xd.device, _lib.lib().bs_workspace_bytes(I, M, N, 16, T))
+    ws[:ws.numel() // 4 * 4].view(torch.float32).fill_(float("nan"))
+    y = IU.bitstack_forward_hip(qd, ud, vd, xd).cpu().numpy()
+    assert y.shape == (T, M) and np.isfinite(y).all()
+    assert_close(y, exact, "vs fp64")
+    # token by token through the one-token kernel: the same numbers up to fp32 summation order
+    y1 = torch.cat([IU.bitstack_forward_hip(qd, ud, vd, xd[t:t + 1].contiguous()) for t in range(T)]).float().cpu().numpy()
+    assert np.abs(y.astype(np.float64) - y1).max() <= 2e-3 * np.abs(y1).max()
+
+
 @pytest.mark.parametrize("I,M,N,T,K", [(2, 128, 512, 1, 16), (3, 256, 1024, 2, 5), (2, 64, 512, 1, 1)])
 def test_forward_decode_signed_factors_bias_and_small_rank(I, M, N, T, K):
     print(f"forward signed I={I} M={M} N={N} T={T} K={K}", flush=True)
@@ -276,7 +298,7 @@ def test_full_size_properties_largest_decode_shape():
     rows = [0, 1, 4095, 7777, 14335]
     exact = O.forward_exact(np.stack([qq.cpu().numpy().reshape(M, N // 8)[rows].reshape(-1) for qq in q]),
                             u[:, rows].cpu().numpy(), vt.cpu().numpy(), x.cpu().numpy())
-    assert_close(y[:, rows].cpu().numpy(), exact, "spot rows vs fp64", 1e-2, 2e-3)
+    assert_close(y[:, rows].cpu().numpy(), exact, "spot rows vs fp64", 1e-2, 1e-3)
 
 
 @pytest.mark.parametrize("M,N", [(28672, 8192), (8192, 28672), (8192, 8192), (1024, 8192)])
@@ -297,7 +319,7 @@ def test_llama_70b_shapes_spot_rows_on_every_path(M, N):
         print(f"70B shape M={M} N={N} I={I} T={T}", flush=True)
         y = f(q, u, vt, x[:T].contiguous())
         assert tuple(y.shape) == (T, M)
-        assert_close(y[:, rows].cpu().numpy(), exact[:T], f"T={T} spot rows vs fp64", 1e-2, 2e-3)
+        assert_close(y[:, rows].cpu().numpy(), exact[:T], f"T={T} spot rows vs fp64", 1e-2, 1e-3)
         ys[T] = y.float()
     scale = float(ys[64].abs().max())
     for T in (1, 4, 8):
@@ -515,3 +537,59 @@ def test_forward_random_shapes(I, M, N, T, K):
                                 None if bias is None else bias.to(dev())).cpu().numpy()
     assert y.shape == (T, M)
     assert_close(y, exact, "vs fp64")
+
+
+# ------------------------------------------------------------- beyond 2^31 elements
+def test_unpack_more_than_2_31_signs():
+    """The reference splits its launches above 2^31 - 1 elements (bitstack/utils/pack_utils.py:181-194);
+    here one call with 64-bit indices.  2^31 + 40 signs, compared with numpy.unpackbits on windows at the
+    start, around every multiple of 2^29 elements up to and across the 2^31 boundary, and at the end."""
+    n = (1 << 31) + 40
+    print(f"unpack n={n}", flush=True)
+    g = torch.Generator(device=dev()).manual_seed(31)
+    packed = torch.randint(0, 256, ((n + 7) // 8,), dtype=torch.uint8, device=dev(), generator=g)
+    out = PU.unpack_sign_hip(packed, (n,))
+    assert out.dtype == torch.int8 and out.numel() == n
+    span = 1 << 16                                          # bytes per window
+    starts = [0] + [k * (1 << 26) - span // 2 for k in range(1, 5)] + [packed.numel() - span]
+    for b0 in starts:
+        want = np.unpackbits(packed[b0:b0 + span].cpu().numpy(), bitorder="big").astype(np.int8) * 2 - 1
+        got = out[8 * b0:8 * (b0 + span)].cpu().numpy()
+        assert np.array_equal(got, want[:got.size]), b0
+    # nothing but +-1 anywhere, and as many +1 as there are set bits (a window written twice or skipped
+    # would change the count); summed in slabs to bound the temporaries
+    ones = 0
+    for s0 in range(0, n, 1 << 28):
+        sl = out[s0:s0 + (1 << 28)]
+        assert bool(((sl == 1) | (sl == -1)).all())
+        ones += int((sl == 1).sum())
+    lut = torch.tensor([bin(v).count("1") for v in range(256)], device=dev())
+    bits = 0
+    for s0 in range(0, packed.numel(), 1 << 26):
+        bits += int(lut[packed[s0:s0 + (1 << 26)].long()].sum())
+    assert ones == bits
+
+
+def test_forward_with_2_31_weights_takes_the_rebuild_path():
+    """M * N = 2^31: the decode kernel keeps per-block byte offsets in 32 bits and declines; the call must
+    still be right through the rebuilt weight (one block, one token and six)."""
+    I, M, N = 1, 32768, 65536
+    print(f"forward M*N=2^31 I={I} M={M} N={N}", flush=True)
+    assert _lib.decode_plan(I, M, N, 16, 1)[0] == 0
+    g = torch.Generator(device=dev()).manual_seed(7)
+    q = torch.randint(0, 256, (I, M * N // 8), dtype=torch.uint8, device=dev(), generator=g)
+    u = (torch.randn(I, M, 16, device=dev(), generator=g).abs() * 0.01).half()
+    vt = (torch.randn(I, 16, N, device=dev(), generator=g).abs() * 0.01).half()
+    x = torch.randn(6, N, device=dev(), generator=g).half()
+    rows = [0, 1, 16383, 16384, 16385, M - 1]               # rows either side of byte offset 2^27 * 8 and the last one
+    qs = np.stack([qq.view(M, N // 8)[rows].reshape(-1).cpu().numpy() for qq in q])
+    exact = O.forward_exact(qs, u[:, rows].cpu().numpy(), vt.cpu().numpy(), x.cpu().numpy())
+    for T in (1, 6):
+        y = IU.bitstack_forward_hip(q, u, vt, x[:T].contiguous())
+        assert tuple(y.shape) == (T, M)
+        assert_close(y[:, rows].cpu().numpy(), exact[:T], f"T={T} spot rows vs fp64")
+    # the last rows of the weight itself, bit for bit against the C oracle's fp32 rebuild order within one ulp
+    w = IU.unpack_and_reconstruct_w_hip(q, u, vt)
+    tail = C.reconstruct_w(qs[:, -N // 8:].copy(), u[:, M - 1:].cpu().numpy(), vt.cpu().numpy())
+    got = w[M - 1:].cpu().numpy()
+    assert np.all(np.abs(got.astype(np.float64) - tail.astype(np.float64)) <= np.spacing(np.abs(tail)).astype(np.float64))

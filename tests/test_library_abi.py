@@ -141,9 +141,9 @@ def test_no_fallback_when_the_library_or_the_device_is_missing(tmp_path):
     from bitstack_amd.utils import inference_utils as IU
     from bitstack_amd.utils import pack_utils as PU
     code = ("import bitstack_amd._lib as L\n"
+            f"L.LIB_PATH = {str(tmp_path / 'absent.so')!r}\n"
             "try:\n    L.lib()\nexcept RuntimeError as e:\n    print('RAISED', e)\n")
-    env = dict(os.environ, BITSTACK_AMD_LIB=str(tmp_path / "absent.so"))
-    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env,
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True,
                          cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert "RAISED" in out.stdout and "is missing" in out.stdout and "no fallback" in out.stdout, out.stdout + out.stderr
     q = torch.zeros(2, 64 * 512 // 8, dtype=torch.uint8)

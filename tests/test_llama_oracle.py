@@ -76,3 +76,31 @@ def test_attention_closed_forms():
     out = lo.attention_decode(q, kc, vc, 5)
     assert np.allclose(out[1], vc[0].mean(0)) and np.allclose(out[2], vc[1].mean(0))
     assert np.isclose(lo.silu(0.0), 0.0) and np.isclose(lo.silu(50.0), 50.0) and np.isclose(lo.silu(1.0), 1 / (1 + np.exp(-1.0)))
+
+
+def test_rope_frequencies_with_llama3_scaling_match_transformers():
+    """The decoder's RoPE tables for the released Llama-3.1 / 3.2 configurations (rope_type "llama3")
+    against the library the reference runs those models through; plain and linear scaling too, and
+    an unknown type is refused instead of silently giving default tables."""
+    import pytest
+    from transformers import LlamaConfig
+    from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+    from bitstack_amd.utils.llama_decode import rope_inv_freq
+    for d, theta, sc in [(128, 500000.0, dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                               original_max_position_embeddings=8192)),
+                         (64, 500000.0, dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                              original_max_position_embeddings=8192)),
+                         (64, 10000.0, dict(rope_type="linear", factor=4.0))]:
+        cfg = LlamaConfig(hidden_size=d * 2, num_attention_heads=2, num_hidden_layers=1, intermediate_size=64, vocab_size=8,
+                          head_dim=d, max_position_embeddings=131072, rope_parameters=dict(sc, rope_theta=theta))
+        want, att = ROPE_INIT_FUNCTIONS[sc["rope_type"]](cfg, "cpu")
+        got = rope_inv_freq(d, theta, sc)
+        assert att == 1.0 and got.dtype == torch.float32
+        assert torch.allclose(got, want.float(), rtol=1e-6, atol=0), sc
+        plain = rope_inv_freq(d, theta, None)
+        assert torch.equal(plain[0:1], got[0:1]) or sc["rope_type"] == "linear"     # the fastest frequency is untouched by llama3
+        assert not torch.equal(plain, got)
+    assert torch.allclose(rope_inv_freq(8, 100.0), torch.tensor([1.0, 100 ** -0.25, 100 ** -0.5, 100 ** -0.75]))
+    assert torch.equal(rope_inv_freq(8, 100.0, {"rope_type": "default"}), rope_inv_freq(8, 100.0))
+    with pytest.raises(ValueError, match="yarn"):
+        rope_inv_freq(64, 10000.0, {"rope_type": "yarn", "factor": 2.0})
