@@ -41,9 +41,17 @@ extern "C" int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int
     if (!waves || !row_tiles_per_wave || !workgroups || !partials_per_row) return BS_ERR_NULL;
     int st = forward_dims(I, M, N, K, T);
     if (st != BS_OK) return st;
-    bs_gemv_plan_info(I, M, N, T, waves, row_tiles_per_wave, workgroups, partials_per_row);
+    bs_gemv_plan_info(I, M, N, K, T, waves, row_tiles_per_wave, workgroups, partials_per_row);
     return BS_OK;
 }
+
+extern "C" int bs_decode_kernel(int I, int M, int N, int K, int T) {
+    int st = forward_dims(I, M, N, K, T);
+    if (st != BS_OK) return st;
+    return bs_gemv_plan_kernel(I, M, N, K, T);
+}
+
+extern "C" int bs_set_decode_kernel(int mode) { return bs_gemv_set_kernel(mode); }
 
 extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void *x,
                           const void *bias, void *y, int I, int M, int N, int K, int T,

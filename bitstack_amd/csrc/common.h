@@ -65,7 +65,9 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
                    const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
                    void *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T);
-void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax);
+void bs_gemv_plan_info(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax);
+int bs_gemv_plan_kernel(int I, int M, int N, int K, int T);
+int bs_gemv_set_kernel(int mode);
 // epilogues of the grouped decode forward (values of BS_EPI_* in the public header)
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, int K, int T);

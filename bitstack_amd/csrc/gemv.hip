@@ -50,6 +50,7 @@
 // the epilogue (none, + residual, silu(a) * b): deterministic, no atomics.  Workgroups with neighbouring ranges - which read
 // the same slices of vt - sit on the same XCD (and share its L2).
 #include "common.h"
+#include "gemv_shared.h"
 
 #include <type_traits>
 #include <utility>
@@ -67,6 +68,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 constexpr int CH = 512;   // columns per chunk: 4 lane groups x 16 bytes of signs
+constexpr int64_t MX_MIN_SIGN_BYTES = 12 << 20;   // sign bytes per launch from which the block-scaled kernel is preferred
 
 
 // step -> bit position used in that step; steps 0-7 read the word as loaded,
@@ -130,40 +132,6 @@ __device__ inline void produce_finish(half_t *zt, int pg, int p, int r, half8_t 
         *reinterpret_cast<half2_t *>(zt + z_index(0, st, pg, r) + 2 * p) = o;
     });
 }
-
-// Static partition of U units over G workgroups: the first `rem` get q + 1.
-struct Split {
-    int q, rem;
-    __host__ __device__ int start(int w) const { return w * q + (w < rem ? w : rem); }
-    __host__ __device__ int owner(int unit) const {
-        const int big = rem * (q + 1);
-        return unit < big ? unit / (q + 1) : rem + (unit - big) / q;
-    }
-};
-
-// Up to GEMV_MAX_GROUP matrices that share x (and so N and K) run in one launch:
-// the grid is cut into one run of workgroups per matrix, each with its own static
-// partition, partial-sum area and row count.
-constexpr int GEMV_MAX_GROUP = 4;
-constexpr int GEMV_WIDE_MIN_UNITS = 1024;   // 1024-row units from which one token runs on 16-wave workgroups
-constexpr int GEMV_PAIR_MIN_UNITS = 4;      // units per workgroup from which workgroups are paired
-struct GemvMat {
-    const uint8_t *packed;
-    const half_t *u, *vt;
-    float *part;
-    int M, row_tiles, kmax, first_wg;
-    Split sp;
-    // 1: workgroups 2p and 2p + 1 share one range of (block, row tile, chunk PAIR) units and
-    // take the even / the odd 512-column chunk of every pair.  The two 64-byte halves of a
-    // 128-byte line of sign bytes are then requested at about the same time by neighbours on
-    // one XCD (the second request hits L2) instead of one unit apart by the same workgroup,
-    // by when the line has often been evicted and comes from HBM again.
-    int pair;
-};
-struct GemvGroup {
-    GemvMat m[GEMV_MAX_GROUP];
-    int n;
-};
 
 template <int T, int WAVES, int R>
 __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4 && R == 4 ? 3 : 4) : (T == 2 ? (WAVES == 8 && R == 2 ? 4 : 2) : 1))) void gemv_kernel(
@@ -607,6 +575,7 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
 
 struct Plan {
     int waves, R, n_chunks, grid, n, pair;
+    int mx;        // 1: the block-scaled fp4 x fp6 kernel (gemv_mx.hip), units of MX_UNIT_COLS columns
     int row_tiles[GEMV_MAX_GROUP], kmax[GEMV_MAX_GROUP], first_wg[GEMV_MAX_GROUP];
     Split sp[GEMV_MAX_GROUP];
     int64_t part_off[GEMV_MAX_GROUP];      // in floats; part_off[n] = total
@@ -615,10 +584,77 @@ struct Plan {
 
 // One instantiation and one grid for the whole group; every matrix gets a share of
 // the workgroups in proportion to its units.
-Plan make_plan(const int *I, const int *M, int n, int N, int T) {
+// Which one-token kernel make_plan picks: 0 by shape, 1 always the fp16 kernel, 2 the block-scaled one
+// wherever it takes the shape (bs_set_decode_kernel, for tests and benchmarks).
+int g_decode_kernel = 0;
+
+// Rows per workgroup of the block-scaled kernel for these matrices (0: it does not run them).
+int mx_rows_per_tile(const int *I, const int *M, int n, int N, int K, int T) {
+    if (T != 1 || g_decode_kernel == 1 || !bs_gemv_mx_takes(N, K, 1)) return 0;
+    const int n_units = (int)bs_cdiv(N, MX_UNIT_COLS);
+    int pick = 0;
+    for (int r = 8; r >= 1; r >>= 1) {
+        const int rw = 8 * r * 16;
+        bool tall = true;
+        int64_t units = 0;
+        for (int j = 0; j < n; j++) {
+            tall = tall && M[j] >= rw;
+            units += bs_cdiv(M[j], rw) * I[j] * n_units;
+        }
+        if ((tall && units >= 256) || r == 1) { pick = r; break; }
+    }
+    if (g_decode_kernel == 2) return pick;
+    // by shape: the long-stack cases, where the contraction loop and not the fixed cost of a launch decides
+    int64_t bytes = 0;
+    for (int j = 0; j < n; j++) bytes += (int64_t)I[j] * M[j] * (N / 8);
+    return (pick >= 4 && bytes >= MX_MIN_SIGN_BYTES) ? pick : 0;
+}
+
+Plan make_plan(const int *I, const int *M, int n, int N, int K, int T) {
     Plan p;
     p.n = n;
     p.n_chunks = N / CH;
+    p.mx = 0;
+    const int mx_r = mx_rows_per_tile(I, M, n, N, K, T);
+    if (mx_r > 0) {
+        // one workgroup of 8 waves per CU; units are (block, row tile, 1024 columns), never paired
+        p.mx = 1;
+        p.waves = 8;
+        p.R = mx_r;
+        p.pair = 0;
+        p.n_chunks = (int)bs_cdiv(N, MX_UNIT_COLS);
+        int units[GEMV_MAX_GROUP], total = 0, biggest = 0;
+        for (int j = 0; j < n; j++) {
+            p.row_tiles[j] = (int)bs_cdiv(M[j], 8 * mx_r * 16);
+            units[j] = I[j] * p.row_tiles[j] * p.n_chunks;
+            total += units[j];
+            if (units[j] > units[biggest]) biggest = j;
+        }
+        int grid = total < 256 ? total : 256, gj[GEMV_MAX_GROUP], sum = 0;
+        for (int j = 0; j < n; j++) {
+            gj[j] = n == 1 ? grid : (int)(((int64_t)grid * units[j] + total / 2) / total);
+            if (gj[j] < 1) gj[j] = 1;
+            if (gj[j] > units[j]) gj[j] = units[j];
+            sum += gj[j];
+        }
+        while (sum > grid && gj[biggest] > 1) { gj[biggest]--; sum--; }
+        int first = 0;
+        int64_t off = 0;
+        for (int j = 0; j < n; j++) {
+            p.first_wg[j] = first;
+            first += gj[j];
+            p.sp[j].q = units[j] / gj[j];
+            p.sp[j].rem = units[j] % gj[j];
+            int kmax = (int)bs_cdiv(p.n_chunks - 1, p.sp[j].q) + 1;
+            if (kmax > gj[j]) kmax = gj[j];
+            p.kmax[j] = kmax;
+            p.part_off[j] = off;
+            off += (int64_t)I[j] * kmax * T * M[j];
+        }
+        p.grid = first;
+        p.part_total = off;
+        return p;
+    }
     // rows per workgroup: 512 (8 waves x 4 tiles), 256, 128, 64; resident workgroups per CU.
     // Three or four tokens need more than the 128 registers a lane has with two 8-wave
     // workgroups per CU: there it is one workgroup of 8 waves per CU (two waves per SIMD
@@ -874,7 +910,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
     float *part = (float *)workspace;
     for (int t0 = 0; t0 < T; t0 += tp) {
         const int tn = (T - t0 < tp) ? T - t0 : tp;
-        const Plan p = make_plan(a.I, a.M, a.n, N, tn);
+        const Plan p = make_plan(a.I, a.M, a.n, N, K, tn);
         if (!workspace || workspace_bytes < p.part_total * (int64_t)sizeof(float)) return BS_ERR_WORKSPACE;
         GemvGroup g;
         RedGroup r;
@@ -897,7 +933,8 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         const half_t *xp = x + (int64_t)t0 * N;
         r.xin = input_rms ? xp : nullptr;
         int st;
-        switch (tn) {
+        if (p.mx) st = bs_launch_gemv_mx(p.R, p.grid, g, xp, N, K, p.n_chunks, s);
+        else switch (tn) {
             case 1: st = launch_T<1>(p, g, xp, N, K, s); break;
             case 2: st = launch_T<2>(p, g, xp, N, K, s); break;
             case 3: st = launch_T<3>(p, g, xp, N, K, s); break;
@@ -913,11 +950,11 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
 }
 
 // Scratch the factor-through path needs: the largest partial area over its passes.
-int64_t gemv_part_floats(const int *I, const int *M, int n, int N, int T) {
+int64_t gemv_part_floats(const int *I, const int *M, int n, int N, int K, int T) {
     const int tp = pass_tokens(T), tail = T % tp;
-    int64_t need = make_plan(I, M, n, N, tp).part_total;
+    int64_t need = make_plan(I, M, n, N, K, tp).part_total;
     if (tail) {
-        const int64_t t2 = make_plan(I, M, n, N, tail).part_total;
+        const int64_t t2 = make_plan(I, M, n, N, K, tail).part_total;
         if (t2 > need) need = t2;
     }
     return need;
@@ -935,19 +972,31 @@ int64_t bs_gemv_group_workspace_bytes(const int *I, const int *M, int n, int N, 
     const int path = group_path(I, M, n, N, K, T);
     if (path < 0) return 0;
     if (path == 1) return strip_part_floats(I, M, n, N, K, T) * (int64_t)sizeof(float);
-    return gemv_part_floats(I, M, n, N, T) * (int64_t)sizeof(float);
+    return gemv_part_floats(I, M, n, N, K, T) * (int64_t)sizeof(float);
 }
 
 // Which instantiation and grid a decode forward of these dimensions runs
 // (0 in *waves when the decode kernel does not take them).
-void bs_gemv_plan_info(int I, int M, int N, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax) {
+void bs_gemv_plan_info(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax) {
     *waves = *row_tiles_per_wave = *grid = *kmax = 0;
-    if (group_path(&I, &M, 1, N, 16, T) != 0) return;
-    const Plan p = make_plan(&I, &M, 1, N, pass_tokens(T));
+    if (group_path(&I, &M, 1, N, K, T) != 0) return;
+    const Plan p = make_plan(&I, &M, 1, N, K, pass_tokens(T));
     *waves = p.waves;
     *row_tiles_per_wave = p.R;
     *grid = p.grid;
     *kmax = p.kmax[0];
+}
+
+// 0: not a decode-kernel shape, 1: gemv_kernel (fp16 MFMA), 2: gemv_mx_kernel (block-scaled fp4 x fp6 MFMA)
+int bs_gemv_plan_kernel(int I, int M, int N, int K, int T) {
+    if (group_path(&I, &M, 1, N, K, T) != 0) return 0;
+    return make_plan(&I, &M, 1, N, K, pass_tokens(T)).mx ? 2 : 1;
+}
+
+int bs_gemv_set_kernel(int mode) {
+    if (mode < 0 || mode > 2) return BS_ERR_SHAPE;
+    g_decode_kernel = mode;
+    return BS_OK;
 }
 
 // Returns BS_ERR_SHAPE when the fast path does not apply (the caller falls

@@ -1,0 +1,436 @@
+// One-token packed-sign GEMV on the block-scaled MFMA of gfx950
+// (v_mfma_scale_f32_16x16x128_f8f6f4): signs as the fp4 operand, Z = vt o x as fp6.
+//
+//   y[m] = sum_i sum_r u_i[m, r] * ( sum_n s_i[m, n] * Z_i[r, n] ),   Z_i[r, n] = vt_i[r, n] * x[n]
+//
+// Same contraction as gemv_kernel (D[r, m] += Z[r, n] S[m, n] on the matrix cores, 16 MACs per
+// sign bit), but one MFMA now takes K = 128 columns and both operands come cheap:
+//
+// ---- the sign operand: one VALU instruction per EIGHT signs -----------------------------
+// An fp4 (e2m1) operand register holds eight 4-bit codes.  A lane keeps its 16 bytes of signs
+// (128 columns of one row) as loaded; MFMA number q = 3..0 of those columns uses bit q of every
+// nibble, so its four operand registers are `word & (0x11111111 << q)`, nothing else:
+//     q = 3   the fp4 sign bit, merged with the code of 1.0: (w & 0x88888888) | 0x22222222 = -+1
+//             (bit set = code -1.0 although it means +1: Z enters negated for these columns)
+//     q = 2   code 0100 = 2.0 or 0           B scale 1   value 1 + s
+//     q = 1   code 0010 = 1.0 or 0           B scale 2   value 1 + s
+//     q = 0   code 0001 = 0.5 or 0           B scale 4   value 1 + s
+// so for q < 3 the MFMA accumulates sum (1 + s) z = sum z + sum s z.  The first sum does not
+// depend on the row: the wave that produced the Z operand adds it up with one extra MFMA per
+// term against the constant operand 1.0, and the shares are exchanged through LDS at flush time
+// and subtracted (exactly: the same quantised z on both sides).
+// Nibble e of word p of a lane in lane group g is column 128 g + 8 (4 p + e / 2) + (e odd ? 3 - q
+// : 7 - q) of the lane's 512-column half unit: the Z operand is produced in that order.
+//
+// ---- the Z operand: three fp6 terms with block scales -----------------------------------
+// z = vt * x is formed in fp16 (as gemv_kernel does), then split per (rank, 32 columns of one
+// MFMA lane) into z = t1 2^e1 + t2 2^(e1-4) + t3 2^(e1-8) + rest with t_k in e2m3, by the
+// hardware conversion v_cvt_scalef32_pk32_fp6_f16 (32 halves -> 32 packed fp6, round to nearest)
+// and its inverse: t1 = cvt(z / 2^e1), r1 = z - t1 2^e1 (exact in fp16), t2 = cvt(r1 / 2^(e1-4)),
+// ...  e1 puts the block maximum in [3.75, 7.5] (the top of e2m3), so |r1| <= 2^e1 / 4,
+// |r2| <= 2^e1 / 128, |rest| <= 2^(e1-12): under 7e-5 of the block maximum, a fifth of the fp16
+// rounding z already carries.  The three terms are three MFMAs into one accumulator, their
+// scales the three low bytes of one E8M0 scale register.
+//
+// A unit is (block, row tile of 8 * R * 16 rows, 1024 columns): both 64-byte halves of every
+// 128-byte line of sign bytes are requested back to back by the same lane.  Z for the next unit
+// is produced by all 512 threads, one (half, q, rank, lane group) operand each.
+#include "gemv_shared.h"
+
+#include <type_traits>
+#include <utility>
+
+namespace {
+
+typedef int v8i_t __attribute__((ext_vector_type(8)));
+typedef unsigned v6u_t __attribute__((ext_vector_type(6)));
+typedef _Float16 half32_t __attribute__((ext_vector_type(32)));
+
+constexpr int MX_WAVES = 8;
+constexpr int MX_OPERAND = 64 * 16 + 64 * 8;        // bytes of one (half, q, term) operand: dwords 0-3, then dwords 4-5, per lane
+constexpr int MX_SCALES = 8 * 3 * MX_OPERAND;       // the scale words of a Z buffer follow its 24 operands
+constexpr int MX_ZBUF = MX_SCALES + 8 * 64 * 4;     // bytes per Z buffer
+
+__device__ __forceinline__ float4_t mx_mfma(const uint4_t &a03, const uint2_t &a45, const uint4_t &b, float4_t c,
+                                            int term, uint32_t scale_a, uint32_t scale_b) {
+    const v8i_t av = {(int)a03[0], (int)a03[1], (int)a03[2], (int)a03[3], (int)a45[0], (int)a45[1], 0, 0};
+    const v8i_t bv = {(int)b[0], (int)b[1], (int)b[2], (int)b[3], 0, 0, 0, 0};
+    // A fp6 e2m3 (cbsz 2), B fp4 e2m1 (blgp 4); the A scale is byte `term` of scale_a
+    switch (term) {
+        case 0: return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 2, 4, 0, (int)scale_a, 0, (int)scale_b);
+        case 1: return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 2, 4, 1, (int)scale_a, 0, (int)scale_b);
+        default: return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, c, 2, 4, 2, (int)scale_a, 0, (int)scale_b);
+    }
+}
+
+// Production of the Z operands of one half unit (512 columns) for FOUR ranks by one wave: every vt
+// value of a unit is loaded exactly once per workgroup, by coalesced 16-byte loads (load k is rank
+// 4 j + k, lane l the 8 columns 8 l .. 8 l + 7 of the half unit; x likewise, one piece per lane).
+// Of a piece's 8 products, position q uses columns 7 - q and 3 - q (negated for q = 3).  The pairs
+// go through a transpose in a staging area private to the wave, so that lane (rank k', group g',
+// position q') ends up with the 32 values z[2 b + hh], b = 0..15, of ONE MFMA operand lane; those
+// are split into three fp6 terms and written where consumer lane 16 g' + rank reads them.
+constexpr int MX_STAGE_BLK = 20;                     // dwords per staged (rank, position, group) block: 16 + 4, so that the
+                                                     // 16-byte reads of 8 consecutive lanes hit 8 different bank groups
+constexpr int MX_STAGE = 64 * MX_STAGE_BLK * 4;      // bytes of staging per wave
+__device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, const half8_t (&pv)[4], const half8_t &px,
+                                                  int h, int j, int lane, int K) {
+    {
+        const int g = lane >> 4, b = lane & 15;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            half8_t p = pv[k] * px;
+            if (4 * j + k >= K) p = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                half2_t pr = {p[7 - q], p[3 - q]};
+                if (q == 3) pr = -pr;
+                stage[((k * 4 + q) * 4 + g) * MX_STAGE_BLK + b] = __builtin_bit_cast(uint32_t, pr);
+            }
+        }
+    }
+    // the reads below are of another type than the stores above: keep the compiler from moving them up
+    // (the LDS operations of one wave execute in order, so no wait is needed)
+    asm volatile("" ::: "memory");
+    const int k = lane & 3, g = (lane >> 2) & 3, q = lane >> 4;
+    uint4_t zw[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) zw[e] = *reinterpret_cast<const uint4_t *>(stage + ((k * 4 + q) * 4 + g) * MX_STAGE_BLK + 4 * e);
+    half32_t z;
+    half2_t mx = {(half_t)0, (half_t)0};
+#pragma unroll
+    for (int b = 0; b < 16; b++) {
+        const uint32_t word = zw[b >> 2][b & 3];      // (a bit cast applied to the element expression itself reads element 0)
+        const half2_t v = __builtin_bit_cast(half2_t, word);
+        z[2 * b] = v[0];
+        z[2 * b + 1] = v[1];
+        mx = __builtin_elementwise_max(mx, __builtin_elementwise_abs(v));
+    }
+    const float m = fmaxf((float)mx[0], (float)mx[1]);
+    // exponent of s1 = floor(log2(m * 16 / 15)) - 2: the conversions use the exponent only
+    const float s1 = fmaxf(m * (4.f / 15.f), 0x1p-100f), s2 = s1 * 0x1p-4f, s3 = s1 * 0x1p-8f;
+    const uint32_t e1 = __builtin_bit_cast(uint32_t, s1) >> 23;
+    const uint32_t scale = e1 | ((e1 - 4u) << 8) | ((e1 - 8u) << 16);
+    const v6u_t t1 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(z, s1);
+    const half32_t r1 = z - __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t1, s1);
+    const v6u_t t2 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(r1, s2);
+    const half32_t r2 = r1 - __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t2, s2);
+    const v6u_t t3 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(r2, s3);
+    const int hq = 4 * h + q, cl = 16 * g + 4 * j + k;             // operand set and consumer lane this thread feeds
+    char *op = zbuf + hq * 3 * MX_OPERAND;
+    *reinterpret_cast<uint4_t *>(op + cl * 16) = (uint4_t){t1[0], t1[1], t1[2], t1[3]};
+    *reinterpret_cast<uint2_t *>(op + 1024 + cl * 8) = (uint2_t){t1[4], t1[5]};
+    *reinterpret_cast<uint4_t *>(op + MX_OPERAND + cl * 16) = (uint4_t){t2[0], t2[1], t2[2], t2[3]};
+    *reinterpret_cast<uint2_t *>(op + MX_OPERAND + 1024 + cl * 8) = (uint2_t){t2[4], t2[5]};
+    *reinterpret_cast<uint4_t *>(op + 2 * MX_OPERAND + cl * 16) = (uint4_t){t3[0], t3[1], t3[2], t3[3]};
+    *reinterpret_cast<uint2_t *>(op + 2 * MX_OPERAND + 1024 + cl * 8) = (uint2_t){t3[4], t3[5]};
+    *reinterpret_cast<uint32_t *>(zbuf + MX_SCALES + hq * 256 + cl * 4) = scale;
+}
+
+template <int R>
+__global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
+    const GemvGroup grp, const half_t *__restrict__ x, int N, int K, int n_units) {
+    constexpr int RW = MX_WAVES * R * 16;          // rows per workgroup
+    constexpr int TG = R < 4 ? R : 4;              // row tiles whose sign operands are live together
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    char *zl = lds;                                                            // [2][MX_ZBUF]
+    float *corrl = reinterpret_cast<float *>(lds + 2 * MX_ZBUF + MX_WAVES * MX_STAGE);   // [2][MX_WAVES][16]
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lm = lane & 15, g = lane >> 4;
+
+    // XCD-aware slot -> range (workgroups are dealt round-robin to the 8 XCDs; each XCD gets a
+    // contiguous run of ranges), then the matrix of the group this workgroup belongs to
+    int wg;
+    {
+        const int nb = gridDim.x, xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+        const int base = nb >> 3, rem = nb & 7;
+        wg = xcd * base + min(xcd, rem) + loc;
+    }
+    GemvMat mat = grp.m[0];
+#pragma unroll
+    for (int j = 1; j < GEMV_MAX_GROUP; j++)
+        if (j < grp.n && wg >= grp.m[j].first_wg) mat = grp.m[j];
+    wg -= mat.first_wg;
+    const uint8_t *__restrict__ packed = mat.packed;
+    const half_t *__restrict__ u = mat.u;
+    const half_t *__restrict__ vt = mat.vt;
+    float *__restrict__ part = mat.part;
+    const int M = mat.M, row_tiles = mat.row_tiles, kmax = mat.kmax;
+    const Split sp = mat.sp;
+    const int u_begin = sp.start(wg), u_end = sp.start(wg + 1);
+    if (u_begin >= u_end) return;
+
+    const int64_t row_bytes = N >> 3;
+    // producer role: half unit wave / 4, ranks 4 (wave % 4) .. + 3
+    const int ph = wave >> 2, pj = wave & 3;
+    uint32_t *stage = reinterpret_cast<uint32_t *>(lds + 2 * MX_ZBUF + wave * MX_STAGE);
+
+    // a unit whose second half lies beyond N (N a multiple of 512 only) reads the first half's
+    // addresses again there; x counts as zero for those columns, so they add nothing
+    auto half_cols = [&](int c, int h) { return (c * MX_UNIT_COLS + 512 * h < N) ? 512 * h : 0; };
+
+    // ---- the unit being loaded: (block li, row tile, 1024-column chunk lc) ------------------------
+    // Sign words and vt pieces are requested for the unit AFTER the one being multiplied; `qoff`,
+    // `lq`, `lv` always describe that unit.
+    uint32_t qoff[R];           // this lane's row in each row tile of the wave, as a byte offset within a block
+    const uint8_t *lq;          // packed signs of the block, at the unit's first column
+    const half_t *lv;           // vt of the block: rank 4 pj, this lane's 8 columns of half ph of the unit
+    int l_h1;                   // byte offset of the unit's second half of a row (0 when it lies beyond N)
+    bool l_xlive;               // the producer half of this wave lies within N
+    auto set_unit = [&](int rowid, int c, bool new_row) {
+        const int i = rowid / row_tiles;
+        if (new_row) {
+            const int rt = rowid - i * row_tiles;
+#pragma unroll
+            for (int jr = 0; jr < R; jr++) {
+                const uint32_t row = (uint32_t)min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
+                qoff[jr] = row * (uint32_t)row_bytes + 16u * g;
+            }
+        }
+#ifdef MXEXP_SAME_SIGNS
+        lq = packed + (c & 1) * (MX_UNIT_COLS >> 3);
+#else
+        lq = packed + (int64_t)i * M * row_bytes + c * (MX_UNIT_COLS >> 3);
+#endif
+        l_h1 = half_cols(c, 1) >> 3;
+        lv = vt + ((int64_t)i * K + 4 * pj) * N + c * MX_UNIT_COLS + half_cols(c, ph) + 8 * lane;    // (4 pj may exceed K - 1: see produce_issue)
+        l_xlive = c * MX_UNIT_COLS + 512 * ph < N;
+    };
+
+    float4_t acc[R];
+    float4_t corr;
+    auto clear_acc = [&]() {
+        corr = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jr = 0; jr < R; jr++) acc[jr] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    };
+    clear_acc();
+
+    half8_t pv[4], px;          // in flight: vt of rank 4 pj + k and x, columns 8 lane .. 8 lane + 7 of this wave's half unit
+    auto produce_issue = [&](int c) {
+        // (ranks beyond K repeat rank K - 1 and are zeroed when the operands are formed: no branch around a load)
+#pragma unroll
+        for (int k = 0; k < 4; k++) pv[k] = *reinterpret_cast<const half8_t *>(lv + (int64_t)(min(4 * pj + k, K - 1) - 4 * pj) * N);
+        px = *reinterpret_cast<const half8_t *>(x + c * MX_UNIT_COLS + half_cols(c, ph) + 8 * lane);
+    };
+    auto produce_write = [&](int buf) {
+        if (!l_xlive) px = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
+        mx_produce_finish(zl + buf * MX_ZBUF, stage, pv, px, ph, pj, lane, K);
+    };
+
+    // ---- one (half, position) pass: per row tile four ANDs and three MFMAs ---------------------------
+    // The sign words of a half unit are used by its four passes; in the last of them (q = 3, the
+    // sign position, whose codes need the OR) every word is re-requested for the next unit right
+    // behind its last use, so the sign bytes need one register set, not two.  (Unconditionally: a
+    // branch around a load makes the compiler keep both values and wait for everything in flight.)
+    uint4_t w[R][2];
+    auto pass = [&](const uint4_t &p0, const uint4_t &p1, const uint4_t &p2, const uint2_t &r0, const uint2_t &r1,
+                    const uint2_t &r2, uint32_t sa, auto hq_const) {
+        constexpr int h = decltype(hq_const)::value >> 2, q = decltype(hq_const)::value & 3;
+        constexpr uint32_t ONES = 0x22222222u;           // 1.0 in every nibble
+        constexpr uint32_t mask = 0x11111111u << q;
+        // B scale that makes a set bit worth 2 (q < 3: codes 2, 1, 0.5) or the sign code worth 1
+        constexpr uint32_t sb = q == 3 ? 127u : 129u - q;
+#pragma unroll
+        for (int j0 = 0; j0 < R; j0 += TG) {
+            uint4_t b[TG];
+#pragma unroll
+            for (int jr = 0; jr < TG; jr++) {
+#pragma unroll
+                for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? ((w[j0 + jr][h][p] & mask) | ONES) : (w[j0 + jr][h][p] & mask);
+                if (q == 3) w[j0 + jr][h] = *reinterpret_cast<const uint4_t *>(lq + qoff[j0 + jr] + (h ? l_h1 : 0));
+            }
+            // term by term over the row tiles: consecutive MFMAs never share an accumulator
+#pragma unroll
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p0, r0, b[jr], acc[j0 + jr], 0, sa, sb);
+#pragma unroll
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p1, r1, b[jr], acc[j0 + jr], 1, sa, sb);
+#pragma unroll
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p2, r2, b[jr], acc[j0 + jr], 2, sa, sb);
+            // pin the products to this pass: the optimiser otherwise sinks all MFMAs of a unit below the
+            // operand reads of all its passes (the scheduling fences bind the instruction scheduler only)
+#pragma unroll
+            for (int jr = 0; jr < TG; jr++) asm volatile("" : "+v"(acc[j0 + jr]));
+        }
+    };
+    // The three fp6 terms of this lane's Z operand for a pass (dwords 0-3 and 4-5 of each) and their scale
+    // word, in two register sets: operands are fetched one pass ahead.  Plain variables and explicit
+    // passes: kept in a struct, or left to the unroller, they end up in scratch memory or all in
+    // registers at once; the scheduling fences keep the eight passes apart.
+#define MX_FETCH(S, HQ)                                                                                            \
+    do {                                                                                                           \
+        const char *op_ = zbuf + (HQ) * 3 * MX_OPERAND;                                                            \
+        S##p0 = *reinterpret_cast<const uint4_t *>(op_ + lane * 16);                                               \
+        S##r0 = *reinterpret_cast<const uint2_t *>(op_ + 1024 + lane * 8);                                         \
+        S##p1 = *reinterpret_cast<const uint4_t *>(op_ + MX_OPERAND + lane * 16);                                  \
+        S##r1 = *reinterpret_cast<const uint2_t *>(op_ + MX_OPERAND + 1024 + lane * 8);                            \
+        S##p2 = *reinterpret_cast<const uint4_t *>(op_ + 2 * MX_OPERAND + lane * 16);                              \
+        S##r2 = *reinterpret_cast<const uint2_t *>(op_ + 2 * MX_OPERAND + 1024 + lane * 8);                        \
+        S##sa = *reinterpret_cast<const uint32_t *>(zbuf + MX_SCALES + (HQ) * 256 + lane * 4);                     \
+    } while (0)
+#define MX_PASS(S, HQ)                                                                                             \
+    do {                                                                                                           \
+        pass(S##p0, S##p1, S##p2, S##r0, S##r1, S##r2, S##sa, std::integral_constant<int, HQ>{});                   \
+        __builtin_amdgcn_sched_barrier(0);                                                                         \
+    } while (0)
+    auto consume = [&](int buf) {
+        const char *zbuf = zl + buf * MX_ZBUF;
+        uint4_t fa_p0, fa_p1, fa_p2, fb_p0, fb_p1, fb_p2;
+        uint2_t fa_r0, fa_r1, fa_r2, fb_r0, fb_r1, fb_r2;
+        uint32_t fa_sa, fb_sa;
+        MX_FETCH(fa_, 0);
+        MX_FETCH(fb_, 1);
+        MX_PASS(fa_, 0);
+        MX_FETCH(fa_, 2);
+        MX_PASS(fb_, 1);
+        MX_FETCH(fb_, 3);
+        MX_PASS(fa_, 2);
+        MX_FETCH(fa_, 4);
+        MX_PASS(fb_, 3);
+        MX_FETCH(fb_, 5);
+        MX_PASS(fa_, 4);
+        MX_FETCH(fa_, 6);
+        MX_PASS(fb_, 5);
+        MX_FETCH(fb_, 7);
+        MX_PASS(fa_, 6);
+        MX_PASS(fb_, 7);
+        // For the positions whose codes are 1 + s the accumulators also hold the sum of z over the
+        // position's columns.  It does not depend on the row: wave w adds it up for operand set w
+        // (one MFMA per term against the constant operand 1.0), the shares meet at flush time.
+        if ((wave & 3) != 3) {
+            constexpr uint32_t ONES = 0x22222222u;
+            const uint4_t ones = {ONES, ONES, ONES, ONES};
+            MX_FETCH(fa_, wave);
+            corr = mx_mfma(fa_p0, fa_r0, ones, corr, 0, fa_sa, 127u);
+            corr = mx_mfma(fa_p1, fa_r1, ones, corr, 1, fa_sa, 127u);
+            corr = mx_mfma(fa_p2, fa_r2, ones, corr, 2, fa_sa, 127u);
+        }
+    };
+#undef MX_FETCH
+#undef MX_PASS
+
+    // D[r, m]: the lane holds ranks 4g..4g+3 of row (tile jr, lm).  Subtract the correction
+    // (summed over waves in a fixed order), scale by u, add the four lane groups, write the
+    // partial row sum, start the next row from zero.
+    int flush_parity = 0;
+    auto flush = [&](int rowid) {
+        // two flushes can follow each other with no barrier in between, so the exchange area alternates
+        float *cx = corrl + flush_parity * (MX_WAVES * 16);
+        flush_parity ^= 1;
+        const int i = rowid / row_tiles, rt = rowid % row_tiles;
+        half4_t uc[R];
+#pragma unroll
+        for (int jr = 0; jr < R; jr++) {
+            const int row = min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
+            const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
+            if (K == 16) {
+                uc[jr] = *reinterpret_cast<const half4_t *>(up);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; v++) uc[jr][v] = (4 * g + v < K) ? up[v] : (half_t)0;
+            }
+        }
+        if (lm == 0) *reinterpret_cast<float4_t *>(cx + wave * 16 + 4 * g) = corr;
+        __syncthreads();
+        const int slot = wg - sp.owner(rowid * n_units);
+        float4_t cz = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ww = 0; ww < MX_WAVES; ww++) cz += *reinterpret_cast<const float4_t *>(cx + ww * 16 + 4 * g);
+#pragma unroll
+        for (int jr = 0; jr < R; jr++) {
+            const int row = rt * RW + (wave * R + jr) * 16 + lm;
+            float val = (acc[jr][0] - cz[0]) * (float)uc[jr][0] + (acc[jr][1] - cz[1]) * (float)uc[jr][1] +
+                        (acc[jr][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][3] - cz[3]) * (float)uc[jr][3];
+            val += __shfl_xor(val, 16, 64);
+            val += __shfl_xor(val, 32, 64);
+            if (g == 0 && row < M) part[((int64_t)i * kmax + slot) * M + row] = val;
+        }
+        clear_acc();
+    };
+
+    // ---- pipeline fill: first unit's signs and Z ----------------------------------------------
+    int rowid = u_begin / n_units, c = u_begin % n_units;
+    set_unit(rowid, c, true);
+    produce_issue(c);
+#pragma unroll
+    for (int jr = 0; jr < R; jr++) {
+        w[jr][0] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr]);
+        w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
+    }
+    uint32_t warm0;      // loaded for its side effect only (the line ends up in L2)
+    {
+        const int lrow = (u_end - 1) / n_units, fi = lrow / row_tiles, frt = lrow % row_tiles;
+        const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
+        warm0 = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
+    }
+    produce_write(0);
+    __syncthreads();
+    asm volatile("" ::"v"(warm0));
+
+    // ---- steady state ----------------------------------------------------------------------------
+    int buf = 0;
+    uint32_t warm_in = 0;
+    for (int unit = u_begin; unit + 1 < u_end; unit++) {
+        const bool crossing = c + 1 == n_units;     // the next unit starts another row of units
+        const int cn = crossing ? 0 : c + 1;
+        if (crossing) {
+            // the row ends with this unit: pull its u rows towards L2 now (one dword per row, value unused)
+            const int fi = rowid / row_tiles, frt = rowid % row_tiles;
+            const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
+            warm_in = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
+        }
+        set_unit(rowid + (crossing ? 1 : 0), cn, crossing);
+#ifndef MXEXP_NO_PRODUCE
+        produce_issue(cn);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+        consume(buf);
+        asm volatile("" ::"v"(warm_in));
+#ifndef MXEXP_NO_PRODUCE
+        produce_write(buf ^ 1);
+#endif
+        __syncthreads();
+        if (crossing) {
+            flush(rowid);
+            rowid++;
+        }
+        c = cn;
+        buf ^= 1;
+    }
+    // ---- drain ---------------------------------------------------------------------------------------
+    consume(buf);          // (its refill requests repeat the last unit's addresses: valid, unused)
+    flush(rowid);
+}
+
+size_t mx_lds_bytes() { return (size_t)2 * MX_ZBUF + (size_t)MX_WAVES * MX_STAGE + 2 * MX_WAVES * 16 * sizeof(float); }
+
+template <int R>
+int launch_mx(int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
+    const size_t lds = mx_lds_bytes();
+    static bs_lds_grant granted[BS_MAX_DEVICES];
+    const int st = bs_allow_lds((const void *)gemv_mx_kernel<R>, lds, granted);
+    if (st != BS_OK) return st;
+    gemv_mx_kernel<R><<<grid, 64 * MX_WAVES, lds, s>>>(grp, x, N, K, n_units);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
+}  // namespace
+
+// Shapes the block-scaled kernel runs: whole 512-column halves.
+bool bs_gemv_mx_takes(int N, int K, int R) {
+    if (N % 512 != 0 || K < 1 || K > 16) return false;
+    return R == 1 || R == 2 || R == 4 || R == 8;
+}
+
+int bs_launch_gemv_mx(int R, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
+    if (!bs_gemv_mx_takes(N, K, R) || n_units != (int)bs_cdiv(N, MX_UNIT_COLS)) return BS_ERR_SHAPE;
+    switch (R) {
+        case 1: return launch_mx<1>(grid, grp, x, N, K, n_units, s);
+        case 2: return launch_mx<2>(grid, grp, x, N, K, n_units, s);
+        case 4: return launch_mx<4>(grid, grp, x, N, K, n_units, s);
+        default: return launch_mx<8>(grid, grp, x, N, K, n_units, s);
+    }
+}
