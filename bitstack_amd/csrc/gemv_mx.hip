@@ -354,11 +354,11 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     int rowid = u_begin / n_units, c = u_begin % n_units;
     set_unit(rowid, c, true);
     produce_issue(c);
+    // first halves first: the first four passes need nothing else (requests complete in order)
 #pragma unroll
-    for (int jr = 0; jr < R; jr++) {
-        w[jr][0] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr]);
-        w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
-    }
+    for (int jr = 0; jr < R; jr++) w[jr][0] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr]);
+#pragma unroll
+    for (int jr = 0; jr < R; jr++) w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
     uint32_t warm0;      // loaded for its side effect only (the line ends up in L2)
     {
         const int lrow = (u_end - 1) / n_units, fi = lrow / row_tiles, frt = lrow % row_tiles;
