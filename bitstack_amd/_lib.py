@@ -27,12 +27,14 @@ SIGNATURES = {
     "bs_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
     "bs_decode_plan": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _P]),
     "bs_forward": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _L, _P]),
+    "bs_forward_static": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "bs_linear_f16": (_I, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "bs_linear_plan": (_I, [_I, _I, _I, _P, _P, _P, _P]),
     "bs_decode_kernel": (_I, [_I, _I, _I, _I, _I]),
     "bs_set_decode_kernel": (_I, [_I]),
 }
 DECODE_AUTO, DECODE_F16, DECODE_MX = 0, 1, 2
+STATIC_SCRATCH_BYTES = 64 << 20
 
 
 

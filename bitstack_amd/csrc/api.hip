@@ -1,6 +1,8 @@
 // C ABI glue: argument validation, path selection, status strings.
 #include "common.h"
 
+#include <mutex>
+
 extern "C" int bs_version(void) { return BS_VERSION_NUMBER; }
 
 extern "C" const char *bs_error_string(int status) {
@@ -78,6 +80,47 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     st = bs_launch_reconstruct_packed(packed, (const half_t *)u, (const half_t *)vt, w, I, M, N, K, s);
     if (st != BS_OK) return st;
     return bs_launch_linear_f16((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N, s);
+}
+
+// ---- the forward for callers that cannot allocate ------------------------------------
+// The scratch of the decode and strip kernels (partial row sums) lives in a file-scope device
+// array instead of a caller-owned workspace.  Every GPU the library runs on holds its own copy
+// of the array at its own address until the process ends; `scratch` itself is only the
+// host-side handle of the symbol, so the address is looked up once per device (with that
+// device current) and only the looked-up pointer is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[BS_STATIC_SCRATCH_BYTES];
+static void *g_scratch_ptr[BS_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void **out) {
+    int dev = -1;
+    BS_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= BS_MAX_DEVICES) return BS_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        BS_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return BS_ERR_NO_DEVICE;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return BS_OK;
+}
+
+extern "C" int bs_forward_static(const uint8_t *packed, const void *u, const void *vt, const void *x,
+                                 const void *bias, void *y, int I, int M, int N, int K, int T, void *stream) {
+    int st = forward_dims(I, M, N, K, T);
+    if (st != BS_OK) return st;
+    if (T == 0) return BS_OK;
+    // sizes first: a call that would not fit is refused before any device is touched
+    const int64_t need = bs_workspace_bytes(I, M, N, K, T);
+    if (need < 0) return (int)need;
+    if (need > (int64_t)BS_STATIC_SCRATCH_BYTES) return BS_ERR_WORKSPACE;
+    void *ws = nullptr;
+    st = static_scratch(&ws);
+    if (st != BS_OK) return st;
+    // nothing in the scratch has to start at zero: every partial sum a call reads it has written before
+    return bs_forward(packed, u, vt, x, bias, y, I, M, N, K, T, ws, (int64_t)BS_STATIC_SCRATCH_BYTES, stream);
 }
 
 // ---- grouped decode forward ---------------------------------------------------

@@ -108,6 +108,26 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
                void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * bs_forward for callers that cannot allocate device memory or pass a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  The scratch of the kernels is a
+ * device array inside the library, BS_STATIC_SCRATCH_BYTES per GPU, held until
+ * the process ends; the call allocates nothing and frees nothing.  Dimensions
+ * whose bs_workspace_bytes exceeds BS_STATIC_SCRATCH_BYTES return
+ * BS_ERR_WORKSPACE: 64 MiB holds the partial sums of every 1..4-token forward of
+ * the 8B and 70B linear shapes up to 36 blocks and of their 5..8-token forwards
+ * up to 12 blocks; the strip kernel at several dozen tokens on the largest
+ * matrices and every forward that rebuilds a weight of more than 32 Mi elements
+ * (more than 48 tokens, or N not a multiple of 128) need more and are refused.
+ * All calls on one GPU share the one array: calls that overlap in time on the
+ * same GPU (different streams, different host threads) race; calls on one
+ * stream are ordered and safe.  Same results as bs_forward, bit for bit.
+ */
+#define BS_STATIC_SCRATCH_BYTES (64 << 20)
+int bs_forward_static(const uint8_t *packed, const void *u, const void *vt, const void *x,
+                      const void *bias, void *y, int I, int M, int N, int K, int T, void *stream);
+
+/*
  * Introspection for benchmarks and tests: which decode kernel instantiation
  * (waves per workgroup, 16-row tiles per wave), how many workgroups and how
  * many partial sums per row and block bs_forward would use for these
