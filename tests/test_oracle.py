@@ -250,3 +250,29 @@ def test_retrieve_compression_config():
     assert O.retrieve_compression_config(cfgs, 100) == {"a": 3}
     with pytest.raises(ValueError):
         O.retrieve_compression_config(cfgs, 2)
+
+
+def test_torch_level0_restatement_matches_the_oracle():
+    """oracle/torch_l0.py (what the CPU baseline of the benchmark times) against the numpy level-0
+    restatement: the same unpack, the same fp16 running sum of the weight, F.linear with fp32
+    accumulation - outputs equal to the last fp16 bit or its neighbour, signs bit for bit."""
+    import torch
+    from oracle import torch_l0
+    rng = np.random.default_rng(12)
+    I, M, N, K, T = 3, 48, 64, 16, 2
+    q = rng.integers(0, 256, size=(I, M * N // 8), dtype=np.uint8)
+    u = (np.abs(rng.standard_normal((I, M, K))) * 0.1).astype(np.float16)
+    vt = (np.abs(rng.standard_normal((I, K, N))) * 0.1).astype(np.float16)
+    x = rng.standard_normal((T, N)).astype(np.float16)
+    bias = rng.standard_normal(M).astype(np.float16)
+    s = torch_l0.unpack_sign(torch.from_numpy(q[0]), torch.Size((M, N))).numpy()
+    assert np.array_equal(s, O.unpack_sign(q[0], (M, N)))
+    for b in (None, bias):
+        got = torch_l0.forward_l0(torch.from_numpy(q), torch.from_numpy(u), torch.from_numpy(vt), torch.from_numpy(x),
+                                  None if b is None else torch.from_numpy(b)).numpy()
+        want = O.forward_l0(q, u, vt, x, b)
+        assert got.dtype == np.float16 and got.shape == want.shape
+        ulp = np.spacing(np.abs(want).astype(np.float16)).astype(np.float64)
+        assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= ulp)
+        exact = O.forward_exact(q, u, vt, x, b)
+        assert np.abs(got - exact).max() <= 1e-2 * np.abs(exact).max()
