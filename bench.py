@@ -38,6 +38,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+PEAK_CLOCK_HZ = 2.4e9         # MI355X peak engine clock
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 BLOCKS = [1, 2, 4, 8, 16]
 PREFILL_T = [16, 128, 512, 2048]
@@ -443,8 +444,8 @@ def main():
     # kernel's launches separates the per-launch cost from the streaming rate; the floors are the HBM time of the
     # bytes and the matrix-core issue time of the contraction (16 MACs per sign bit; the block-scaled kernel issues
     # three 16x16x128 MFMAs of 16 + 4 cycles per 16 x 128 signs, the fp16 kernel four 16x16x32 MFMAs of 16 cycles
-    # per 16 x 128 signs, on 1024 SIMDs at the device's peak clock).
-    clock_hz = torch.cuda.get_device_properties(0).clock_rate * 1e3
+    # per 16 x 128 signs, on 1024 SIMDs at the 2.4 GHz peak clock).
+    clock_hz = PEAK_CLOCK_HZ
     def mfma_floor_us(L):
         tiles = L.I * L.M * L.N / (16.0 * 128.0)
         cycles = tiles * (60.0 if "mx" in dom else 64.0)

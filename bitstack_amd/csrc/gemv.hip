@@ -407,7 +407,8 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
 //   EPI_NONE      the matrices' outputs side by side in one row of `ldy` halves
 //   EPI_RESIDUAL  the same plus residual[t, off + m]
 //   EPI_SWIGLU    two matrices of equal M: silu(first) * second, one row of M
-constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;   // the last one is a sanity limit on the block count
+constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;
+constexpr int RED_BATCH = 4;      // partial loads in flight per thread (eight were slower: the loads of dead slots are issued all the same)   // the last one is a sanity limit on the block count
 
 struct RedMat {
     const float *part;
@@ -433,7 +434,7 @@ struct RedGroup {
 
 // Sum of the partials of output m of one matrix that this thread's slice covers.
 // The (block, slot) pairs are numbered i * kmax + k and slice ks takes every
-// RED_SL-th of them, four at a time: slots that are not live (k beyond the number of
+// RED_SL-th of them, RED_BATCH at a time: slots that are not live (k beyond the number of
 // workgroups that touched this row tile of block i, `nks[i]`, worked out once per
 // workgroup) are loaded all the same (the slots exist in the workspace) and masked, so
 // the loads of a batch never wait for one another.  (i, k) advance incrementally: no
@@ -452,11 +453,11 @@ __device__ __forceinline__ typename RedVec<VEC>::type slice_sum_any(const RedMat
     const float *base = r.part + (int64_t)t * r.M + m;
     vec_t acc = vec_t(0.f);
     int i = ks / r.kmax, k = ks - i * r.kmax;                  // slot ks
-    for (int s0 = ks; s0 < total; s0 += 4 * RED_SL) {
-        vec_t v[4];
-        bool ok[4];
+    for (int s0 = ks; s0 < total; s0 += RED_BATCH * RED_SL) {
+        vec_t v[RED_BATCH];
+        bool ok[RED_BATCH];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < RED_BATCH; j++) {
             const bool in = s0 + j * RED_SL < total;
             const int ic = in ? i : 0, kc = in ? k : 0;
             ok[j] = in && kc < nks[ic];
@@ -465,7 +466,7 @@ __device__ __forceinline__ typename RedVec<VEC>::type slice_sum_any(const RedMat
             while (k >= r.kmax) { k -= r.kmax; i++; }
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc += ok[j] ? v[j] : vec_t(0.f);
+        for (int j = 0; j < RED_BATCH; j++) acc += ok[j] ? v[j] : vec_t(0.f);
     }
     return acc;
 }
