@@ -588,14 +588,13 @@ struct Plan {
 // Which one-token kernel make_plan picks: 0 by shape, 1 always the fp16 kernel, 2 the block-scaled one
 // wherever it takes the shape (bs_set_decode_kernel, for tests and benchmarks).
 int g_decode_kernel = 0;
-int g_decode_force_r = 0;     // experiments: row tiles per wave of the block-scaled kernel (0: by shape)
 
 // Rows per workgroup of the block-scaled kernel for these matrices (0: it does not run them).
 int mx_rows_per_tile(const int *I, const int *M, int n, int N, int K, int T) {
     if (T != 1 || g_decode_kernel == 1 || !bs_gemv_mx_takes(N, K, 1)) return 0;
     const int n_units = (int)bs_cdiv(N, MX_UNIT_COLS);
     int pick = 0;
-    for (int r = g_decode_force_r ? g_decode_force_r : 4; r >= 1; r >>= 1) {
+    for (int r = 4; r >= 1; r >>= 1) {
         const int rw = 8 * r * 16;
         bool tall = true;
         int64_t units = 0;
@@ -996,9 +995,8 @@ int bs_gemv_plan_kernel(int I, int M, int N, int K, int T) {
 }
 
 int bs_gemv_set_kernel(int mode) {
-    if ((mode & 255) > 2) return BS_ERR_SHAPE;
-    g_decode_kernel = mode & 255;
-    g_decode_force_r = mode >> 8;
+    if (mode < 0 || mode > 2) return BS_ERR_SHAPE;
+    g_decode_kernel = mode;
     return BS_OK;
 }
 

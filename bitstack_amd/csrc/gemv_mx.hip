@@ -34,7 +34,15 @@
 //
 // A unit is (block, row tile of 8 * R * 16 rows, 1024 columns): both 64-byte halves of every
 // 128-byte line of sign bytes are requested back to back by the same lane.  Z for the next unit
-// is produced by all 512 threads, one (half, q, rank, lane group) operand each.
+// is produced by all 512 threads while the current one is multiplied: wave w loads four ranks
+// of one 512-column half (every vt value once per workgroup, coalesced), forms the products and
+// passes them through a transpose in LDS to the lanes that convert them, 32 values each.
+//
+// What bounds it (counters and switch-off builds on an MI355X): the scaled MFMA occupies its SIMD
+// for 16 + 4 cycles (matrix pipe + scale load) and VALU work of the other wave on the SIMD does
+// not run underneath it, so a unit costs the SUM of 3 MFMAs (60 cycles) and 4 ANDs (16 cycles)
+// per 16 x 128 signs plus the production of Z (about a third of that at 512 rows per workgroup):
+// about 4.5 TB/s of sign bytes over 256 CUs, before the fill and drain of the pipeline.
 #include "gemv_shared.h"
 
 #include <type_traits>
@@ -189,11 +197,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                 qoff[jr] = row * (uint32_t)row_bytes + 16u * g;
             }
         }
-#ifdef MXEXP_SAME_SIGNS
-        lq = packed + (c & 1) * (MX_UNIT_COLS >> 3);
-#else
         lq = packed + (int64_t)i * M * row_bytes + c * (MX_UNIT_COLS >> 3);
-#endif
         l_h1 = half_cols(c, 1) >> 3;
         lv = vt + ((int64_t)i * K + 4 * pj) * N + c * MX_UNIT_COLS + half_cols(c, ph) + 8 * lane;    // (4 pj may exceed K - 1: see produce_issue)
         l_xlive = c * MX_UNIT_COLS + 512 * ph < N;
@@ -382,15 +386,11 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
             warm_in = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
         }
         set_unit(rowid + (crossing ? 1 : 0), cn, crossing);
-#ifndef MXEXP_NO_PRODUCE
         produce_issue(cn);
-#endif
         __builtin_amdgcn_sched_barrier(0);
         consume(buf);
         asm volatile("" ::"v"(warm_in));
-#ifndef MXEXP_NO_PRODUCE
         produce_write(buf ^ 1);
-#endif
         __syncthreads();
         if (crossing) {
             flush(rowid);
@@ -422,7 +422,7 @@ int launch_mx(int grid, const GemvGroup &grp, const half_t *x, int N, int K, int
 // Shapes the block-scaled kernel runs: whole 512-column halves.
 bool bs_gemv_mx_takes(int N, int K, int R) {
     if (N % 512 != 0 || K < 1 || K > 16) return false;
-    return R == 1 || R == 2 || R == 4 || R == 8;
+    return R == 1 || R == 2 || R == 4;
 }
 
 int bs_launch_gemv_mx(int R, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
@@ -430,7 +430,6 @@ int bs_launch_gemv_mx(int R, int grid, const GemvGroup &grp, const half_t *x, in
     switch (R) {
         case 1: return launch_mx<1>(grid, grp, x, N, K, n_units, s);
         case 2: return launch_mx<2>(grid, grp, x, N, K, n_units, s);
-        case 4: return launch_mx<4>(grid, grp, x, N, K, n_units, s);
-        default: return launch_mx<8>(grid, grp, x, N, K, n_units, s);
+        default: return launch_mx<4>(grid, grp, x, N, K, n_units, s);
     }
 }
