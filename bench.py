@@ -51,7 +51,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
-    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer", "scoring"], default=None,
+    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer", "scoring", "copy"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..48)")
     ap.add_argument("--prompt-len", type=int, default=2048, help="prompt tokens per sequence of --only decode_70b")
@@ -379,6 +379,16 @@ def main():
                                         "decode_plan": _lib.decode_plan(I, M, N, 16, T),
                                         "decode_kernel": {0: "none", 1: "gemv_kernel (fp16 MFMA)", 2: "gemv_mx_kernel (fp4 x fp6 MFMA)"}[
                                             lib.bs_decode_kernel(I, M, N, 16, T)]}}))
+        return
+    if a.only == "copy":
+        # a plain device-to-device copy of 256 MiB, five times: what the FETCH_SIZE / WRITE_SIZE counters read for a
+        # known number of bytes (the calibration of the traffic figures under profiles/)
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy": {"bytes_read": src.numel(), "bytes_written": dst.numel(), "copies": 5}}))
         return
     if a.only == "decode_8b":
         print(json.dumps({"decode_8b": e2e_decode(torch, dev)}))
