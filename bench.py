@@ -299,9 +299,9 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
-    def time_sweep(layers, steps, warmup, per_layer_events):
-        ws = workspace_for(layers)
-        fns = [make_forward(L, lib, ws, stream) for L in layers]
+    def time_fns(fns, steps, warmup, per_layer_events):
+        """The callables in turn, `steps` passes after `warmup` untimed ones: wall clock of the timed
+        passes and, with events around every call, the mean time of each callable (ms)."""
         for _ in range(warmup):
             for f in fns:
                 f()
@@ -326,6 +326,10 @@ def main():
                          for j in range(len(fns))]          # ms per forward
         return wall, per_layer
 
+    def time_sweep(layers, steps, warmup, per_layer_events):
+        ws = workspace_for(layers)
+        return time_fns([make_forward(L, lib, ws, stream) for L in layers], steps, warmup, per_layer_events)
+
     def prefill_side(detail):
         pre = {}
         for T in PREFILL_T:
@@ -336,21 +340,19 @@ def main():
             pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
                             "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
             if T >= 512:
-                # beside it, the module's level 3 on the same layers: this library's rebuild kernel, then
-                # torch's F.linear (hipBLASLt) as in the reference's levels 2-4; never the headline
+                # beside it, timed the same way (the four layers in turn, events around each call):
+                # the same forwards with this library's own dense kernel forced, and the module's level 3 =
+                # this library's rebuild kernel, then torch's F.linear (hipBLASLt) as in the reference's
+                # levels 2-4; never the headline
                 import torch.nn.functional as F
                 from bitstack_amd.utils.inference_utils import unpack_and_reconstruct_w_hip
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                t3 = 0.0
-                for L in lp:
-                    for r in range(4):
-                        if r == 1:
-                            e0.record()
-                        F.linear(L.x, unpack_and_reconstruct_w_hip(L.q, L.u, L.vt))
-                    e1.record()
-                    torch.cuda.synchronize()
-                    t3 += e0.elapsed_time(e1) / 3 * 1e-3
-                pre[f"T{T}"]["level3_rebuild_plus_torch_linear_useful_tflops"] = round(useful / t3 / 1e12, 1)
+                lib.bs_set_dense_kernel(_lib.DENSE_OWN)
+                _, own = time_sweep(lp, 3, 1, per_layer_events=True)
+                lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
+                pre[f"T{T}"]["own_dense_kernel_useful_tflops"] = round(useful / (sum(own) * 1e-3) / 1e12, 1)
+                _, lvl3 = time_fns([(lambda L=L: F.linear(L.x, unpack_and_reconstruct_w_hip(L.q, L.u, L.vt))) for L in lp],
+                                   3, 1, per_layer_events=True)
+                pre[f"T{T}"]["level3_rebuild_plus_torch_linear_useful_tflops"] = round(useful / (sum(lvl3) * 1e-3) / 1e12, 1)
             detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
                         "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
                        for L, ms in zip(lp, perp)]

@@ -32,8 +32,10 @@ SIGNATURES = {
     "bs_linear_plan": (_I, [_I, _I, _I, _P, _P, _P, _P]),
     "bs_decode_kernel": (_I, [_I, _I, _I, _I, _I]),
     "bs_set_decode_kernel": (_I, [_I]),
+    "bs_set_dense_kernel": (_I, [_I]),
 }
 DECODE_AUTO, DECODE_F16, DECODE_MX = 0, 1, 2
+DENSE_AUTO, DENSE_OWN, DENSE_LIBRARY = 0, 1, 2
 STATIC_SCRATCH_BYTES = 64 << 20
 
 

@@ -29,13 +29,33 @@ static int forward_dims(int I, int M, int N, int K, int T) {
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// Which kernel multiplies the rebuilt weight: 0 by token count, 1 always linear_f16_kernel, 2 hipBLASLt
+// wherever it takes the shape (bs_set_dense_kernel, for tests and benchmarks).
+static int g_dense_kernel = 0;
+// From this many tokens on the library's kernels are the faster ones on the layer shapes measured (1024 x 4096 ..
+// 14336 x 4096 with 8 blocks, rebuild included, the four layers run in turn): 384 -> 399 useful TFLOP/s at 512
+// tokens, 662 -> 840 at 2048; at 128 and 256 tokens neither is ahead on every shape.
+constexpr int DENSE_LIBRARY_MIN_T = 512;
+
+static bool dense_wants_library(int M, int N, int T) {
+    if (g_dense_kernel == BS_DENSE_OWN || M % 8 != 0 || N % 8 != 0) return false;
+    return g_dense_kernel == BS_DENSE_LIBRARY || T >= DENSE_LIBRARY_MIN_T;
+}
+
+extern "C" int bs_set_dense_kernel(int mode) {
+    if (mode < 0 || mode > 2) return BS_ERR_SHAPE;
+    g_dense_kernel = mode;
+    return BS_OK;
+}
+
 extern "C" int64_t bs_workspace_bytes(int I, int M, int N, int K, int T) {
     int st = forward_dims(I, M, N, K, T);
     if (st != BS_OK) return st;
     if (T == 0) return 0;
     int64_t gemv = bs_gemv_workspace_bytes(I, M, N, K, T);
     if (gemv > 0) return round_up(gemv, 256);
-    return round_up((int64_t)M * N * 2, 256);
+    // the rebuilt weight, then the library GEMM's own scratch where that is the kernel
+    return round_up((int64_t)M * N * 2, 256) + (dense_wants_library(M, N, T) ? BS_DENSE_LIBRARY_WORKSPACE : 0);
 }
 
 extern "C" int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave,
@@ -79,6 +99,11 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     half_t *w = (half_t *)workspace;
     st = bs_launch_reconstruct_packed(packed, (const half_t *)u, (const half_t *)vt, w, I, M, N, K, s);
     if (st != BS_OK) return st;
+    if (dense_wants_library(M, N, T)) {
+        st = bs_launch_linear_library((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N,
+                                      (char *)workspace + round_up((int64_t)M * N * 2, 256), s);
+        if (st != BS_ERR_SHAPE) return st;      // enqueued, or failed for good; BS_ERR_SHAPE: not for this call
+    }
     return bs_launch_linear_f16((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N, s);
 }
 

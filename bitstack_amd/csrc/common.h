@@ -61,6 +61,10 @@ int bs_launch_reconstruct_packed(const uint8_t *packed, const half_t *u, const h
                                  half_t *w, int I, int M, int N, int K, hipStream_t s);
 int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, half_t *y,
                          int T, int M, int N, hipStream_t s);
+// the same product through hipBLASLt (dense_lt.hip); BS_ERR_SHAPE = not available for this call
+constexpr int64_t BS_DENSE_LIBRARY_WORKSPACE = 64 << 20;
+int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bias, half_t *y, int T, int M, int N,
+                             void *workspace, hipStream_t s);
 int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, const half_t *x,
                    const half_t *bias, half_t *y, int I, int M, int N, int K, int T,
                    void *workspace, int64_t workspace_bytes, hipStream_t s);

@@ -161,6 +161,25 @@ int bs_decode_kernel(int I, int M, int N, int K, int T);
 int bs_set_decode_kernel(int mode);
 
 /*
+ * Test and benchmark hook: which kernel multiplies the rebuilt weight in
+ * bs_forward's large-T path.  0 = by token count (the default: this library's
+ * linear_f16 kernels below 512 tokens, hipBLASLt from there on),
+ * BS_DENSE_OWN = always this library's kernels, BS_DENSE_LIBRARY = hipBLASLt
+ * wherever it takes the shape (M and N multiples of 8).  hipBLASLt is opened
+ * at run time; where it is missing or has no kernel for a shape the call runs
+ * this library's kernel.  bs_workspace_bytes follows the setting (the library
+ * GEMM gets 64 MiB of scratch behind the rebuilt weight).  The first call for
+ * a shape sets the library up (host work, possibly allocations): make it
+ * outside stream capture.  Process-wide and not synchronised, like
+ * bs_set_decode_kernel.  In the reference this product is F.linear on the
+ * rebuilt weight (bitstack/modules/BitStackLinear.py:132,140,148), which on
+ * ROCm is the same library.
+ */
+#define BS_DENSE_OWN     1
+#define BS_DENSE_LIBRARY 2
+int bs_set_dense_kernel(int mode);
+
+/*
  * y[T, M] = x[T, N] @ w[M, N]^T (+ bias) on MFMA, fp32 accumulation: the
  * dense contraction bs_forward uses for large T, exposed for levels 2-4 where
  * the reference calls F.linear on the rebuilt weight

@@ -20,6 +20,14 @@ def dev():
     return torch.device("cuda:0")
 
 
+@pytest.fixture(params=[_lib.DENSE_OWN, _lib.DENSE_LIBRARY], ids=["own_kernel", "hipblaslt"])
+def dense_kernel(request):
+    """bs_forward's large-T path with this library's dense kernel, then with hipBLASLt, behind the same rebuild."""
+    assert _lib.lib().bs_set_dense_kernel(request.param) == 0
+    yield request.param
+    assert _lib.lib().bs_set_dense_kernel(_lib.DENSE_AUTO) == 0
+
+
 def rel(got, ref):
     got, ref = got.double(), ref.double()
     d = (got - ref).abs()
@@ -97,7 +105,7 @@ def spot_rows_exact(q, u, vt, x, rows, bias=None):
 
 @pytest.mark.parametrize("T", [512, 2048])
 @pytest.mark.parametrize("M,N", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
-def test_forward_prefill_8b_shapes_8_blocks(M, N, T):
+def test_forward_prefill_8b_shapes_8_blocks(M, N, T, dense_kernel):
     """Prefill / batched contraction on the 8B shapes with 8 blocks, 512 and 2048 tokens: sampled rows
     against the float64 closed form at the stated tolerance, the whole output against the vendor GEMM on
     the same rebuilt weight, and sub-blocks against the small dense tile."""
@@ -123,7 +131,7 @@ def test_forward_prefill_8b_shapes_8_blocks(M, N, T):
 
 
 @pytest.mark.parametrize("M,N,I", [(8192, 8192, 3), (28672, 8192, 2)])
-def test_forward_prefill_70b_shape_16384_tokens(M, N, I):
+def test_forward_prefill_70b_shape_16384_tokens(M, N, I, dense_kernel):
     """The 70B configuration's prompt pass: every linear sees 2048 x 8 = 16384 tokens at once."""
     T = 16384
     print(f"prefill 70B shape M={M} N={N} I={I} T={T} tile={_lib.linear_plan(T, M, N)}", flush=True)
@@ -142,3 +150,104 @@ def test_forward_prefill_70b_shape_16384_tokens(M, N, I):
     mx, mn = rel(y, vendor)
     print(f"  vs F.linear on the rebuilt weight: max_rel={mx:.3e} mean_rel={mn:.3e}", flush=True)
     assert mx <= 2e-3 and mn <= 2e-4
+
+
+def forward_with(mode, q, u, vt, x, bias=None):
+    lib = _lib.lib()
+    assert lib.bs_set_dense_kernel(mode) == 0
+    try:
+        return IU.bitstack_forward_hip(q, u, vt, x, bias)
+    finally:
+        assert lib.bs_set_dense_kernel(_lib.DENSE_AUTO) == 0
+
+
+# (blocks, out features, in features, tokens, bias): ragged tokens, bias epilogue, a token count below and
+# above the switch-over, out features that are no multiple of 8 (the library path declines: own kernel)
+LIBRARY_CASES = [
+    (3, 4096, 4096, 2047, True),
+    (2, 1024, 4096, 300, False),
+    (2, 14336, 4096, 769, True),
+    (1, 4096, 1536, 1000, False),
+    (2, 4100, 4096, 1024, True),
+    (2, 4099, 4096, 1024, True),
+]
+
+
+@pytest.mark.parametrize("I,M,N,T,with_bias", LIBRARY_CASES)
+def test_forward_library_gemm_matches_own_kernel_and_fp64(I, M, N, T, with_bias):
+    """The hipBLASLt product behind the rebuild against this library's dense kernel on the same call (both
+    round one fp32 sum per output to fp16: all but last-bit ties agree) and sampled rows against float64."""
+    print(f"library gemm I={I} M={M} N={N} T={T} bias={with_bias}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=I + M + T, device=dev())
+    bias = (torch.randn(M, device=dev()) * 0.05).half() if with_bias else None
+    own = forward_with(_lib.DENSE_OWN, q, u, vt, x, bias)
+    got = forward_with(_lib.DENSE_LIBRARY, q, u, vt, x, bias)
+    assert got.dtype == torch.float16 and tuple(got.shape) == (T, M)
+    assert torch.equal(forward_with(_lib.DENSE_LIBRARY, q, u, vt, x, bias), got)
+    mx, mn = rel(got, own)
+    print(f"  vs own kernel: max_rel={mx:.3e} mean_rel={mn:.3e} differing={float((got != own).float().mean()):.2e}", flush=True)
+    assert mx <= 1e-3 and mn <= 5e-5 and float((got != own).float().mean()) < 0.05
+    rows = [0, 1, M // 2, M - 2, M - 1]
+    exact = spot_rows_exact(q, u, vt, x, rows, bias)
+    mx, mn = rel(got[:, rows].cpu(), torch.from_numpy(exact))
+    print(f"  spot rows vs fp64: max_rel={mx:.3e} mean_rel={mn:.3e}", flush=True)
+    assert mx <= MAX_REL and mn <= MEAN_REL
+
+
+def test_dense_kernel_setting_moves_the_workspace_size_and_rejects_unknown_modes():
+    lib = _lib.lib()
+    I, M, N, K = 4, 4096, 4096, 16
+    weight = M * N * 2
+    try:
+        assert lib.bs_set_dense_kernel(_lib.DENSE_OWN) == 0
+        assert lib.bs_workspace_bytes(I, M, N, K, 2048) == weight
+        assert lib.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
+        assert lib.bs_workspace_bytes(I, M, N, K, 2048) == weight + (64 << 20)
+        assert lib.bs_workspace_bytes(I, M, N, K, 100) == weight + (64 << 20)
+        assert lib.bs_workspace_bytes(I, M + 1, N, K, 2048) == (M + 1) * N * 2       # M % 8 != 0: never the library
+        assert lib.bs_workspace_bytes(I, M, N, K, 1) < weight                        # decode shapes do not rebuild
+        assert lib.bs_set_dense_kernel(_lib.DENSE_AUTO) == 0
+        assert lib.bs_workspace_bytes(I, M, N, K, 511) == weight
+        assert lib.bs_workspace_bytes(I, M, N, K, 512) == weight + (64 << 20)
+        assert lib.bs_set_dense_kernel(3) < 0 and lib.bs_set_dense_kernel(-1) < 0
+    finally:
+        lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
+
+
+def test_forward_library_gemm_under_graph_replay():
+    """A captured forward through the library GEMM replays to the eager result every time (the first, eager
+    call has set the library up: the capture only records launches)."""
+    I, M, N, T = 2, 4096, 4096, 1024
+    lib = _lib.lib()
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=5, device=dev())
+    assert lib.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
+    try:
+        need = int(lib.bs_workspace_bytes(I, M, N, 16, T))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev())
+        y = torch.empty((T, M), dtype=torch.float16, device=dev())
+
+        def call(stream):
+            st = lib.bs_forward(_lib.ptr(q), _lib.ptr(u), _lib.ptr(vt), _lib.ptr(x), None, _lib.ptr(y), I, M, N, 16, T,
+                                _lib.ptr(ws), need, stream)
+            assert st == 0, st
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            call(_lib.stream_ptr(dev()))
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        eager = y.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            call(_lib.stream_ptr(dev()))
+        for r in range(3):
+            y.zero_()
+            x2 = x * (1.0 + r)                      # eager work and a synchronisation between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager), r
+            del x2
+    finally:
+        lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
