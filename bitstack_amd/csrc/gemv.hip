@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
     // correction (summed over waves in a fixed order), scale by u, add the four
     // lane groups, write the partial row sum, start the next row from zero.
     int flush_parity = 0;
-    auto flush = [&](int rowid) {
+    auto flush = [&](int rowid, bool row_done) {
         // Two flushes can follow each other with no barrier in between (a row that
         // ends on the last prefetching unit, then the drain), so the exchange area
         // alternates: a wave still reading the previous sums is never overwritten.
@@ -337,7 +337,14 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
                             (acc[jr][t][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][t][3] - cz[3]) * (float)uc[jr][3];
                 val += __shfl_xor(val, 16, 64);
                 val += __shfl_xor(val, 32, 64);
-                if (g == 0 && row < M) part[(((int64_t)i * kmax + slot) * T + t) * M + row] = val;
+                if (g == 0 && row < M) {
+                    part[(((int64_t)i * kmax + slot) * T + t) * M + row] = val;
+                    // The workgroup that finishes a row of units holds its highest live slot: it fills the
+                    // slots nobody writes with zeros, so the summing kernel adds all kmax slots blindly.
+                    if (row_done)
+                        for (int dead = slot + (1 << pair); dead < kmax; dead += 1 << pair)
+                            part[(((int64_t)i * kmax + dead) * T + t) * M + row] = 0.f;
+                }
             }
         }
         clear_acc();
@@ -385,7 +392,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
         produce_write(buf ^ 1);
         __syncthreads();
         if (crossing) {
-            flush(rowid);
+            flush(rowid, true);
             rowid++;
         }
 #pragma unroll
@@ -395,7 +402,7 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
     }
     // ---- drain: last unit, nothing left to prefetch -----------------------------
     consume(cur, buf);
-    flush(rowid);
+    flush(rowid, u_end % nch == 0);
 }
 
 // y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ) where k
@@ -572,6 +579,110 @@ __global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
             y[(int64_t)t * ldy + r.y_off + m + e] = v;
         }
     }
+}
+
+// The same sums for the decode kernels' partials, where EVERY slot of a row holds a number (live
+// partials, zeros in the slots nobody needed): no slot counts, no divisions, and the loads of a thread
+// depend on nothing but its index, so the kernel is one memory round trip long.  A workgroup produces
+// 256 / SL consecutive outputs of one token; SL threads per output take every SL-th of the I * kmax
+// slots (SL = 1: no LDS, no barrier).  SCALED: the input RMS scale of RedGroup::xin.
+constexpr int FLAT_BATCH = 8;
+template <int SL>
+__device__ __forceinline__ float flat_slice_sum(const RedMat &r, int T, int t, int m, int ks) {
+    const int total = r.I * r.kmax;
+    const int64_t stride = (int64_t)T * r.M;
+    const float *base = r.part + (int64_t)t * r.M + m;
+    float acc = 0.f;
+    for (int s0 = ks; s0 < total; s0 += FLAT_BATCH * SL) {
+        float v[FLAT_BATCH];
+#pragma unroll
+        for (int j = 0; j < FLAT_BATCH; j++) {
+            const int s = s0 + j * SL;
+            v[j] = base[(int64_t)(s < total ? s : 0) * stride];
+        }
+#pragma unroll
+        for (int j = 0; j < FLAT_BATCH; j++) acc += (s0 + j * SL < total) ? v[j] : 0.f;
+    }
+    return acc;
+}
+
+template <int SL, bool SCALED>
+__global__ __launch_bounds__(256) void gemv_reduce_flat_kernel(
+    const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy) {
+    constexpr int RUN = 256 / SL;
+    __shared__ float red[2][SL][RUN];
+    __shared__ float ssq[4];
+    const int lo = threadIdx.x % RUN, ks = threadIdx.x / RUN;
+    const bool two = grp.mode == EPI_SWIGLU;
+    int j = 0;
+    if (!two) {
+#pragma unroll
+        for (int q = 1; q < GEMV_MAX_GROUP; q++)
+            if (q < grp.n && (int)blockIdx.x >= grp.m[q].first_block) j = q;
+    }
+    const RedMat &r = grp.m[j];
+    const int local = blockIdx.x - r.first_block;
+    const int per_t = (r.M + RUN - 1) / RUN;
+    const int t = local / per_t, m = (local - t * per_t) * RUN + lo;
+    const bool live = m < r.M;
+    // everything this thread reads is requested before anything is waited for
+    float s0 = live ? flat_slice_sum<SL>(r, T, t, m, ks) : 0.f;
+    float s1 = (two && live) ? flat_slice_sum<SL>(grp.m[1], T, t, m, ks) : 0.f;
+    float extra0 = 0.f, extra1 = 0.f, res = 0.f;
+    if (ks == 0 && live) {
+        if (r.bias) extra0 = (float)r.bias[m];
+        if (two && grp.m[1].bias) extra1 = (float)grp.m[1].bias[m];
+        if (grp.mode == EPI_RESIDUAL) res = (float)residual[(int64_t)t * ldy + r.y_off + m];
+    }
+    float scale = 1.f;
+    if (SCALED) {
+        float q = 0.f;
+        const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
+        for (int c = threadIdx.x * 8; c < grp.n_in; c += 256 * 8) {
+            const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
+#pragma unroll
+            for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o, 64);
+        if ((threadIdx.x & 63) == 0) ssq[threadIdx.x >> 6] = q;
+    }
+    if (SL > 1) {
+        red[0][ks][lo] = s0;
+        if (two) red[1][ks][lo] = s1;
+    }
+    if (SL > 1 || SCALED) __syncthreads();
+    if (SCALED) scale = rsqrtf((ssq[0] + ssq[1] + ssq[2] + ssq[3]) / (float)grp.n_in + grp.eps);
+    if (ks != 0 || !live) return;
+    if (SL > 1) {
+        s0 = 0.f;
+        s1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < SL; k++) s0 += red[0][k][lo];
+        if (two) {
+#pragma unroll
+            for (int k = 0; k < SL; k++) s1 += red[1][k][lo];
+        }
+    }
+    const float a0 = s0 * scale + extra0;
+    if (two) {
+        const float a1 = s1 * scale + extra1;
+        const float gate = (float)(half_t)a0, up = (float)(half_t)a1;
+        const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
+        y[(int64_t)t * ldy + m] = (half_t)((float)act * up);
+    } else {
+        half_t v = (half_t)a0;
+        if (grp.mode == EPI_RESIDUAL) v = (half_t)(res + (float)v);
+        y[(int64_t)t * ldy + r.y_off + m] = v;
+    }
+}
+
+template <int SL>
+void launch_reduce_flat(int blocks, const RedGroup &r, const half_t *residual, half_t *y, int T, int ldy, hipStream_t s) {
+    if (r.xin)
+        gemv_reduce_flat_kernel<SL, true><<<blocks, 256, 0, s>>>(r, residual, y, T, ldy);
+    else
+        gemv_reduce_flat_kernel<SL, false><<<blocks, 256, 0, s>>>(r, residual, y, T, ldy);
 }
 
 struct Plan {
@@ -921,6 +1032,12 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         r.eps = eps;
         r.ssq = nullptr;
         r.ssq_n = 0;
+        // threads per output of the summing kernel: at most FLAT_BATCH loads in flight per thread where the slots allow
+        int slots = 0;
+        for (int j = 0; j < a.n; j++)
+            if (a.I[j] * p.kmax[j] > slots) slots = a.I[j] * p.kmax[j];
+        const int sl = slots <= FLAT_BATCH ? 1 : slots <= 2 * FLAT_BATCH ? 2 : slots <= 4 * FLAT_BATCH ? 4 : 8;
+        const int run = 256 / sl;
         int y_off = 0, blocks = 0;
         for (int j = 0; j < a.n; j++) {
             g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
@@ -928,7 +1045,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
             r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks,
                             p.sp[j], p.pair};
             y_off += a.M[j];
-            if (mode != EPI_SWIGLU || j == 0) blocks += tn * (int)bs_cdiv(a.M[j], RED_OUT);
+            if (mode != EPI_SWIGLU || j == 0) blocks += tn * (int)bs_cdiv(a.M[j], run);
         }
         for (int j = a.n; j < GEMV_MAX_GROUP; j++) { g.m[j] = g.m[0]; r.m[j] = r.m[0]; }
         const half_t *xp = x + (int64_t)t0 * N;
@@ -942,9 +1059,14 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
             default: st = launch_T<4>(p, g, xp, N, K, s); break;
         }
         if (st != BS_OK) return st;
-        gemv_reduce_kernel<1><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual ? residual + (int64_t)t0 * ldy : nullptr,
-                                                               y + (int64_t)t0 * ldy, tn, ldy,
-                                                               p.waves * p.R * 16, p.n_chunks);
+        const half_t *res_p = residual ? residual + (int64_t)t0 * ldy : nullptr;
+        half_t *y_p = y + (int64_t)t0 * ldy;
+        switch (sl) {
+            case 1: launch_reduce_flat<1>(blocks, r, res_p, y_p, tn, ldy, s); break;
+            case 2: launch_reduce_flat<2>(blocks, r, res_p, y_p, tn, ldy, s); break;
+            case 4: launch_reduce_flat<4>(blocks, r, res_p, y_p, tn, ldy, s); break;
+            default: launch_reduce_flat<8>(blocks, r, res_p, y_p, tn, ldy, s); break;
+        }
         BS_LAUNCH_CHECK();
     }
     return BS_OK;

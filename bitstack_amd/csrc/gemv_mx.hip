@@ -319,7 +319,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // (summed over waves in a fixed order), scale by u, add the four lane groups, write the
     // partial row sum, start the next row from zero.
     int flush_parity = 0;
-    auto flush = [&](int rowid) {
+    auto flush = [&](int rowid, bool row_done) {
         // two flushes can follow each other with no barrier in between, so the exchange area alternates
         float *cx = corrl + flush_parity * (MX_WAVES * 16);
         flush_parity ^= 1;
@@ -349,7 +349,13 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                         (acc[jr][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][3] - cz[3]) * (float)uc[jr][3];
             val += __shfl_xor(val, 16, 64);
             val += __shfl_xor(val, 32, 64);
-            if (g == 0 && row < M) part[((int64_t)i * kmax + slot) * M + row] = val;
+            if (g == 0 && row < M) {
+                part[((int64_t)i * kmax + slot) * M + row] = val;
+                // the workgroup that finishes a row of units zero-fills the slots above its own (nobody writes
+                // them): the summing kernel adds all kmax slots blindly
+                if (row_done)
+                    for (int dead = slot + 1; dead < kmax; dead++) part[((int64_t)i * kmax + dead) * M + row] = 0.f;
+            }
         }
         clear_acc();
     };
@@ -393,7 +399,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         produce_write(buf ^ 1);
         __syncthreads();
         if (crossing) {
-            flush(rowid);
+            flush(rowid, true);
             rowid++;
         }
         c = cn;
@@ -401,7 +407,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     }
     // ---- drain ---------------------------------------------------------------------------------------
     consume(buf);          // (its refill requests repeat the last unit's addresses: valid, unused)
-    flush(rowid);
+    flush(rowid, u_end % n_units == 0);
 }
 
 size_t mx_lds_bytes() { return (size_t)2 * MX_ZBUF + (size_t)MX_WAVES * MX_STAGE + 2 * MX_WAVES * 16 * sizeof(float); }
