@@ -493,7 +493,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None if traffic_ratio is None else round(dom_bytes / dom_n * traffic_ratio),
-                     "kernel": dom + " (+ its gemv_reduce_kernel), the instantiation with the most time in the pass",
+                     "kernel": dom + " (+ its gemv_reduce_flat_kernel), the instantiation with the most time in the pass",
                      "launches_per_step": dom_n,
                      "avg_us_per_launch": round(dom_ms * 1e3 / dom_n, 2),
                      "avg_algorithmic_bytes_per_launch": round(dom_bytes / dom_n),

@@ -45,8 +45,10 @@
 // double-buffered LDS image laid out in MFMA operand order: one barrier per
 // unit.  Accumulators are flushed whenever the range crosses into another
 // (block, row tile): scaled by u, reduced over ranks, written as a partial
-// row sum to scratch [I, KMAX, T, M] (fp32).  A second kernel adds the
-// partials of a row in a fixed order, adds the bias, rounds to fp16 and applies
+// row sum to scratch [I, KMAX, T, M] (fp32); the workgroup that ends a row of
+// units also writes zeros to the slots above its own (a row is spread over at
+// most KMAX workgroups, often fewer).  A second kernel adds the KMAX slots of
+// every block in a fixed order, adds the bias, rounds to fp16 and applies
 // the epilogue (none, + residual, silu(a) * b): deterministic, no atomics.  Workgroups with neighbouring ranges - which read
 // the same slices of vt - sit on the same XCD (and share its L2).
 #include "common.h"
