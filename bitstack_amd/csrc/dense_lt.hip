@@ -119,7 +119,9 @@ bool make_plan(LtState &st, hipblasLtHandle_t h, LtPlan &p, int T, int M, int N,
 // BS_OK when the product has been enqueued; BS_ERR_SHAPE when hipBLASLt is not available or has no
 // kernel for the shape (the caller then runs its own).  `workspace` holds BS_DENSE_LIBRARY_WORKSPACE
 // bytes, 256-byte aligned.  The first call for a shape on a device creates the library's handle and
-// asks its heuristic (host work, and the library may allocate): make it outside stream capture.
+// asks its heuristic (host work, and the library may allocate); a shape first seen while its stream is
+// being captured is therefore declined (BS_ERR_SHAPE), and only shapes already run once eagerly are
+// recorded into a graph.
 int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bias, half_t *y, int T, int M, int N,
                              void *workspace, hipStream_t s) {
     if (!bs_aligned(x, 16) || !bs_aligned(w, 16) || !bs_aligned(y, 16) || N % 8 != 0 || M % 8 != 0) return BS_ERR_SHAPE;
@@ -128,14 +130,18 @@ int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bia
     if (dev < 0 || dev >= BS_MAX_DEVICES) return BS_ERR_SHAPE;
     LtState &st = g_lt;
     std::lock_guard<std::mutex> lock(st.mu);
-    if (!load_api(st)) return BS_ERR_SHAPE;
-    if (!st.handle[dev] && st.api.create(&st.handle[dev]) != HIPBLAS_STATUS_SUCCESS) {
-        st.handle[dev] = nullptr;
-        return BS_ERR_SHAPE;
-    }
     const auto key = std::make_tuple(dev, T, M, N, bias ? 1 : 0);
     auto it = st.plans.find(key);
     if (it == st.plans.end()) {
+        // Setting the library up (loading it, its handle, the heuristic) is host work that may allocate:
+        // never under stream capture.  A shape first seen while capturing runs the caller's own kernel.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return BS_ERR_SHAPE;
+        if (!load_api(st)) return BS_ERR_SHAPE;
+        if (!st.handle[dev] && st.api.create(&st.handle[dev]) != HIPBLAS_STATUS_SUCCESS) {
+            st.handle[dev] = nullptr;
+            return BS_ERR_SHAPE;
+        }
         LtPlan p;
         p.usable = make_plan(st, st.handle[dev], p, T, M, N, bias != nullptr);
         it = st.plans.emplace(key, p).first;

@@ -169,8 +169,9 @@ int bs_set_decode_kernel(int mode);
  * at run time; where it is missing or has no kernel for a shape the call runs
  * this library's kernel.  bs_workspace_bytes follows the setting (the library
  * GEMM gets 64 MiB of scratch behind the rebuilt weight).  The first call for
- * a shape sets the library up (host work, possibly allocations): make it
- * outside stream capture.  Process-wide and not synchronised, like
+ * a shape sets the library up (host work, possibly allocations); a shape first
+ * seen under stream capture runs this library's kernel instead, so run a shape
+ * once eagerly if the captured graph is to hold the library GEMM.  Process-wide and not synchronised, like
  * bs_set_decode_kernel.  In the reference this product is F.linear on the
  * rebuilt weight (bitstack/modules/BitStackLinear.py:132,140,148), which on
  * ROCm is the same library.

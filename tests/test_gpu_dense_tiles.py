@@ -251,3 +251,35 @@ def test_forward_library_gemm_under_graph_replay():
             del x2
     finally:
         lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
+
+
+def test_library_gemm_is_not_set_up_under_stream_capture():
+    """A shape the library path has never run is captured with this library's own dense kernel (setting
+    hipBLASLt up may allocate, which a capture forbids); the replay equals the eager own-kernel result, and
+    the eager library result for the same shape, set up afterwards, agrees with both."""
+    I, M, N, T = 2, 2048, 1024, 648                      # a shape no other test sends through the library path
+    lib = _lib.lib()
+    q, u, vt, x = synthetic_layer(M, N, I, T, seed=11, device=dev())
+    try:
+        own = forward_with(_lib.DENSE_OWN, q, u, vt, x)   # eager: the rebuild and dense kernels have run once
+        assert lib.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
+        need = int(lib.bs_workspace_bytes(I, M, N, 16, T))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev())
+        y = torch.zeros((T, M), dtype=torch.float16, device=dev())
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            st = lib.bs_forward(_lib.ptr(q), _lib.ptr(u), _lib.ptr(vt), _lib.ptr(x), None, _lib.ptr(y), I, M, N, 16, T,
+                                _lib.ptr(ws), need, _lib.stream_ptr(dev()))
+            assert st == 0, st
+        for r in range(2):
+            y.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, own), r
+        got = IU.bitstack_forward_hip(q, u, vt, x)         # eager, library mode: now the plan is made
+        mx, mn = rel(got, own)
+        assert mx <= 1e-3 and mn <= 5e-5
+    finally:
+        lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
