@@ -21,7 +21,7 @@ Extra objects on the same JSON line:
                 region (events recorded on the stream the kernels run on).
   cpu_baseline  the reference's CPU path (level 0) restated in torch-CPU ops,
                 timed on this host on one pass of the same sweep.
-  t4, t16, prefill   the same sweep at 4 and at 16 tokens, and the prefill configuration
+  t2, t4, t16, prefill   the same sweep at 2, 4 and 16 tokens, and the prefill configuration
                 (I = 8, T in {16, 128, 512, 2048}) as useful TFLOP/s.
   decode_8b     tokens/s of a random-init Llama-3.1-8B-shape decode loop built
                 around the same forward (batch 1, 256 greedy tokens).
@@ -507,6 +507,19 @@ def main():
     }
 
     if not a.no_extras:
+        # ------------------------------------------------------------ T = 2 sweep (block-scaled kernel, 512-column units)
+        l2 = build_sweep(2)
+        _, per2 = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True)
+        b2 = sum(L.bytes for L in l2)
+        t2 = sum(per2) * 1e-3
+        lib.bs_set_decode_kernel(_lib.DECODE_F16)
+        _, per2f = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True)
+        lib.bs_set_decode_kernel(_lib.DECODE_AUTO)
+        out["t2"] = {"GBps": round(b2 / t2 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b2 / t2 / 1e9 / HBM_PEAK_GBS, 2),
+                     "GBps_fp16_kernel_forced": round(b2 / (sum(per2f) * 1e-3) / 1e9, 1)}
+        detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 2, "bytes": L.bytes, "us": round(ms * 1e3, 2),
+                    "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l2, per2)]
+        del l2
         # ------------------------------------------------------------ T = 4 sweep (MFMA-bound side)
         l4 = build_sweep(4)
         _, per4 = time_sweep(l4, max(3, a.steps // 2), 1, per_layer_events=True)

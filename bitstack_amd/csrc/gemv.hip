@@ -698,14 +698,14 @@ struct Plan {
 
 // One instantiation and one grid for the whole group; every matrix gets a share of
 // the workgroups in proportion to its units.
-// Which one-token kernel make_plan picks: 0 by shape, 1 always the fp16 kernel, 2 the block-scaled one
+// Which kernel make_plan picks for one and two tokens: 0 by shape, 1 always the fp16 kernel, 2 the block-scaled one
 // wherever it takes the shape (bs_set_decode_kernel, for tests and benchmarks).
 int g_decode_kernel = 0;
 
 // Rows per workgroup of the block-scaled kernel for these matrices (0: it does not run them).
 int mx_rows_per_tile(const int *I, const int *M, int n, int N, int K, int T) {
-    if (T != 1 || g_decode_kernel == 1 || !bs_gemv_mx_takes(N, K, 1)) return 0;
-    const int n_units = (int)bs_cdiv(N, MX_UNIT_COLS);
+    if (g_decode_kernel == 1 || !bs_gemv_mx_takes(N, K, 1, T)) return 0;
+    const int n_units = (int)bs_cdiv(N, MX_UNIT_COLS / T);
     int pick = 0;
     for (int r = 4; r >= 1; r >>= 1) {
         const int rw = 8 * r * 16;
@@ -736,7 +736,7 @@ Plan make_plan(const int *I, const int *M, int n, int N, int K, int T) {
         p.waves = 8;
         p.R = mx_r;
         p.pair = 0;
-        p.n_chunks = (int)bs_cdiv(N, MX_UNIT_COLS);
+        p.n_chunks = (int)bs_cdiv(N, MX_UNIT_COLS / T);
         int units[GEMV_MAX_GROUP], total = 0, biggest = 0;
         for (int j = 0; j < n; j++) {
             p.row_tiles[j] = (int)bs_cdiv(M[j], 8 * mx_r * 16);
@@ -1053,7 +1053,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         const half_t *xp = x + (int64_t)t0 * N;
         r.xin = input_rms ? xp : nullptr;
         int st;
-        if (p.mx) st = bs_launch_gemv_mx(p.R, p.grid, g, xp, N, K, p.n_chunks, s);
+        if (p.mx) st = bs_launch_gemv_mx(p.R, tn, p.grid, g, xp, N, K, p.n_chunks, s);
         else switch (tn) {
             case 1: st = launch_T<1>(p, g, xp, N, K, s); break;
             case 2: st = launch_T<2>(p, g, xp, N, K, s); break;

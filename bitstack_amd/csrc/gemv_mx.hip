@@ -1,4 +1,4 @@
-// One-token packed-sign GEMV on the block-scaled MFMA of gfx950
+// One- and two-token packed-sign GEMV on the block-scaled MFMA of gfx950
 // (v_mfma_scale_f32_16x16x128_f8f6f4): signs as the fp4 operand, Z = vt o x as fp6.
 //
 //   y[m] = sum_i sum_r u_i[m, r] * ( sum_n s_i[m, n] * Z_i[r, n] ),   Z_i[r, n] = vt_i[r, n] * x[n]
@@ -32,8 +32,9 @@
 // rounding z already carries.  The three terms are three MFMAs into one accumulator, their
 // scales the three low bytes of one E8M0 scale register.
 //
-// A unit is (block, row tile of 8 * R * 16 rows, 1024 columns): both 64-byte halves of every
-// 128-byte line of sign bytes are requested back to back by the same lane.  Z for the next unit
+// A unit is (block, row tile of 8 * R * 16 rows, 1024 columns) - with two tokens 512 columns of
+// both, so that the operand images of a unit stay the same size: both 64-byte halves of every
+// 128-byte line of sign bytes are requested back to back by the same lane (one unit apart with two tokens).  Z for the next unit
 // is produced by all 512 threads while the current one is multiplied: wave w loads four ranks
 // of one 512-column half (every vt value once per workgroup, coalesced), forms the products and
 // passes them through a transpose in LDS to the lanes that convert them, 32 values each.
@@ -135,9 +136,15 @@ __device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, c
     *reinterpret_cast<uint32_t *>(zbuf + MX_SCALES + hq * 256 + cl * 4) = scale;
 }
 
-template <int R>
+// T = 1: a unit is 1024 columns of one token, its two 512-column halves produced by waves 0-3 and 4-7.
+// T = 2: a unit is 512 columns of two tokens, token t produced by waves 4 t .. 4 t + 3; the eight
+// operand sets of a Z buffer are then (token, position) instead of (half, position), everything else -
+// LDS layout, passes, MFMA count per unit - is the same, and one set of sign words feeds both tokens.
+template <int R, int T>
 __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     const GemvGroup grp, const half_t *__restrict__ x, int N, int K, int n_units) {
+    static_assert(T == 1 || T == 2, "one or two tokens");
+    constexpr int UC = MX_UNIT_COLS / T;           // columns per unit
     constexpr int RW = MX_WAVES * R * 16;          // rows per workgroup
     constexpr int TG = R < 4 ? R : 4;              // row tiles whose sign operands are live together
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -171,13 +178,13 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     if (u_begin >= u_end) return;
 
     const int64_t row_bytes = N >> 3;
-    // producer role: half unit wave / 4, ranks 4 (wave % 4) .. + 3
+    // producer role: half unit (T = 1) or token (T = 2) wave / 4, ranks 4 (wave % 4) .. + 3
     const int ph = wave >> 2, pj = wave & 3;
     uint32_t *stage = reinterpret_cast<uint32_t *>(lds + 2 * MX_ZBUF + wave * MX_STAGE);
 
     // a unit whose second half lies beyond N (N a multiple of 512 only) reads the first half's
     // addresses again there; x counts as zero for those columns, so they add nothing
-    auto half_cols = [&](int c, int h) { return (c * MX_UNIT_COLS + 512 * h < N) ? 512 * h : 0; };
+    auto half_cols = [&](int c, int h) { return (T == 1 && c * UC + 512 * h < N) ? 512 * h : 0; };
 
     // ---- the unit being loaded: (block li, row tile, 1024-column chunk lc) ------------------------
     // Sign words and vt pieces are requested for the unit AFTER the one being multiplied; `qoff`,
@@ -197,18 +204,20 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                 qoff[jr] = row * (uint32_t)row_bytes + 16u * g;
             }
         }
-        lq = packed + (int64_t)i * M * row_bytes + c * (MX_UNIT_COLS >> 3);
+        lq = packed + (int64_t)i * M * row_bytes + c * (UC >> 3);
         l_h1 = half_cols(c, 1) >> 3;
-        lv = vt + ((int64_t)i * K + 4 * pj) * N + c * MX_UNIT_COLS + half_cols(c, ph) + 8 * lane;    // (4 pj may exceed K - 1: see produce_issue)
-        l_xlive = c * MX_UNIT_COLS + 512 * ph < N;
+        lv = vt + ((int64_t)i * K + 4 * pj) * N + c * UC + half_cols(c, ph) + 8 * lane;    // (4 pj may exceed K - 1: see produce_issue)
+        l_xlive = T == 2 || c * UC + 512 * ph < N;
     };
 
-    float4_t acc[R];
-    float4_t corr;
+    float4_t acc[R][T];
+    float4_t corr;              // this wave's operand set belongs to one token (T = 2: token wave / 4)
     auto clear_acc = [&]() {
         corr = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int jr = 0; jr < R; jr++) acc[jr] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int jr = 0; jr < R; jr++)
+#pragma unroll
+            for (int t = 0; t < T; t++) acc[jr][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
     };
     clear_acc();
 
@@ -217,7 +226,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         // (ranks beyond K repeat rank K - 1 and are zeroed when the operands are formed: no branch around a load)
 #pragma unroll
         for (int k = 0; k < 4; k++) pv[k] = *reinterpret_cast<const half8_t *>(lv + (int64_t)(min(4 * pj + k, K - 1) - 4 * pj) * N);
-        px = *reinterpret_cast<const half8_t *>(x + c * MX_UNIT_COLS + half_cols(c, ph) + 8 * lane);
+        px = *reinterpret_cast<const half8_t *>(x + (T == 2 ? (int64_t)ph * N : 0) + c * UC + half_cols(c, ph) + 8 * lane);
     };
     auto produce_write = [&](int buf) {
         if (!l_xlive) px = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
@@ -230,9 +239,12 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // behind its last use, so the sign bytes need one register set, not two.  (Unconditionally: a
     // branch around a load makes the compiler keep both values and wait for everything in flight.)
     uint4_t w[R][2];
+    uint4_t bk[R];              // T = 2: the sign operands of a position, made for token 0 and used again for token 1
     auto pass = [&](const uint4_t &p0, const uint4_t &p1, const uint4_t &p2, const uint2_t &r0, const uint2_t &r1,
                     const uint2_t &r2, uint32_t sa, auto hq_const) {
         constexpr int h = decltype(hq_const)::value >> 2, q = decltype(hq_const)::value & 3;
+        constexpr int wi = T == 1 ? h : 0, ti = T == 1 ? 0 : h;      // sign word set and token of this pass
+        constexpr bool last_use = q == 3 && (T == 1 || h == 1);
         constexpr uint32_t ONES = 0x22222222u;           // 1.0 in every nibble
         constexpr uint32_t mask = 0x11111111u << q;
         // B scale that makes a set bit worth 2 (q < 3: codes 2, 1, 0.5) or the sign code worth 1
@@ -242,21 +254,26 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
             uint4_t b[TG];
 #pragma unroll
             for (int jr = 0; jr < TG; jr++) {
+                if (T == 2 && h == 1) {
+                    b[jr] = bk[j0 + jr];
+                } else {
 #pragma unroll
-                for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? ((w[j0 + jr][h][p] & mask) | ONES) : (w[j0 + jr][h][p] & mask);
-                if (q == 3) w[j0 + jr][h] = *reinterpret_cast<const uint4_t *>(lq + qoff[j0 + jr] + (h ? l_h1 : 0));
+                    for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? ((w[j0 + jr][wi][p] & mask) | ONES) : (w[j0 + jr][wi][p] & mask);
+                    if (T == 2) bk[j0 + jr] = b[jr];
+                }
+                if (last_use) w[j0 + jr][wi] = *reinterpret_cast<const uint4_t *>(lq + qoff[j0 + jr] + (wi ? l_h1 : 0));
             }
             // term by term over the row tiles: consecutive MFMAs never share an accumulator
 #pragma unroll
-            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p0, r0, b[jr], acc[j0 + jr], 0, sa, sb);
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr][ti] = mx_mfma(p0, r0, b[jr], acc[j0 + jr][ti], 0, sa, sb);
 #pragma unroll
-            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p1, r1, b[jr], acc[j0 + jr], 1, sa, sb);
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr][ti] = mx_mfma(p1, r1, b[jr], acc[j0 + jr][ti], 1, sa, sb);
 #pragma unroll
-            for (int jr = 0; jr < TG; jr++) acc[j0 + jr] = mx_mfma(p2, r2, b[jr], acc[j0 + jr], 2, sa, sb);
+            for (int jr = 0; jr < TG; jr++) acc[j0 + jr][ti] = mx_mfma(p2, r2, b[jr], acc[j0 + jr][ti], 2, sa, sb);
             // pin the products to this pass: the optimiser otherwise sinks all MFMAs of a unit below the
             // operand reads of all its passes (the scheduling fences bind the instruction scheduler only)
 #pragma unroll
-            for (int jr = 0; jr < TG; jr++) asm volatile("" : "+v"(acc[j0 + jr]));
+            for (int jr = 0; jr < TG; jr++) asm volatile("" : "+v"(acc[j0 + jr][ti]));
         }
     };
     // The three fp6 terms of this lane's Z operand for a pass (dwords 0-3 and 4-5 of each) and their scale
@@ -284,21 +301,25 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         uint4_t fa_p0, fa_p1, fa_p2, fb_p0, fb_p1, fb_p2;
         uint2_t fa_r0, fa_r1, fa_r2, fb_r0, fb_r1, fb_r2;
         uint32_t fa_sa, fb_sa;
+        // operand sets in the order they are multiplied: half by half (T = 1), or position by position with
+        // both tokens of a position back to back (T = 2: set 4 t + q), so the sign operand is formed once
+        constexpr int O1 = T == 1 ? 1 : 4, O2 = T == 1 ? 2 : 1, O3 = T == 1 ? 3 : 5, O4 = T == 1 ? 4 : 2,
+                      O5 = T == 1 ? 5 : 6, O6 = T == 1 ? 6 : 3;
         MX_FETCH(fa_, 0);
-        MX_FETCH(fb_, 1);
+        MX_FETCH(fb_, O1);
         MX_PASS(fa_, 0);
-        MX_FETCH(fa_, 2);
-        MX_PASS(fb_, 1);
-        MX_FETCH(fb_, 3);
-        MX_PASS(fa_, 2);
-        MX_FETCH(fa_, 4);
-        MX_PASS(fb_, 3);
-        MX_FETCH(fb_, 5);
-        MX_PASS(fa_, 4);
-        MX_FETCH(fa_, 6);
-        MX_PASS(fb_, 5);
+        MX_FETCH(fa_, O2);
+        MX_PASS(fb_, O1);
+        MX_FETCH(fb_, O3);
+        MX_PASS(fa_, O2);
+        MX_FETCH(fa_, O4);
+        MX_PASS(fb_, O3);
+        MX_FETCH(fb_, O5);
+        MX_PASS(fa_, O4);
+        MX_FETCH(fa_, O6);
+        MX_PASS(fb_, O5);
         MX_FETCH(fb_, 7);
-        MX_PASS(fa_, 6);
+        MX_PASS(fa_, O6);
         MX_PASS(fb_, 7);
         // For the positions whose codes are 1 + s the accumulators also hold the sum of z over the
         // position's columns.  It does not depend on the row: wave w adds it up for operand set w
@@ -339,22 +360,27 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         if (lm == 0) *reinterpret_cast<float4_t *>(cx + wave * 16 + 4 * g) = corr;
         __syncthreads();
         const int slot = wg - sp.owner(rowid * n_units);
-        float4_t cz = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ww = 0; ww < MX_WAVES; ww++) cz += *reinterpret_cast<const float4_t *>(cx + ww * 16 + 4 * g);
+        for (int t = 0; t < T; t++) {
+            // the corrections of this token: all eight waves' shares (T = 1), or those of waves 4 t .. 4 t + 3
+            float4_t cz = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int jr = 0; jr < R; jr++) {
-            const int row = rt * RW + (wave * R + jr) * 16 + lm;
-            float val = (acc[jr][0] - cz[0]) * (float)uc[jr][0] + (acc[jr][1] - cz[1]) * (float)uc[jr][1] +
-                        (acc[jr][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][3] - cz[3]) * (float)uc[jr][3];
-            val += __shfl_xor(val, 16, 64);
-            val += __shfl_xor(val, 32, 64);
-            if (g == 0 && row < M) {
-                part[((int64_t)i * kmax + slot) * M + row] = val;
-                // the workgroup that finishes a row of units zero-fills the slots above its own (nobody writes
-                // them): the summing kernel adds all kmax slots blindly
-                if (row_done)
-                    for (int dead = slot + 1; dead < kmax; dead++) part[((int64_t)i * kmax + dead) * M + row] = 0.f;
+            for (int ww = 0; ww < MX_WAVES / T; ww++)
+                cz += *reinterpret_cast<const float4_t *>(cx + (t * (MX_WAVES / T) + ww) * 16 + 4 * g);
+#pragma unroll
+            for (int jr = 0; jr < R; jr++) {
+                const int row = rt * RW + (wave * R + jr) * 16 + lm;
+                float val = (acc[jr][t][0] - cz[0]) * (float)uc[jr][0] + (acc[jr][t][1] - cz[1]) * (float)uc[jr][1] +
+                            (acc[jr][t][2] - cz[2]) * (float)uc[jr][2] + (acc[jr][t][3] - cz[3]) * (float)uc[jr][3];
+                val += __shfl_xor(val, 16, 64);
+                val += __shfl_xor(val, 32, 64);
+                if (g == 0 && row < M) {
+                    part[(((int64_t)i * kmax + slot) * T + t) * M + row] = val;
+                    // the workgroup that finishes a row of units zero-fills the slots above its own (nobody writes
+                    // them): the summing kernel adds all kmax slots blindly
+                    if (row_done)
+                        for (int dead = slot + 1; dead < kmax; dead++) part[(((int64_t)i * kmax + dead) * T + t) * M + row] = 0.f;
+                }
             }
         }
         clear_acc();
@@ -367,8 +393,10 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // first halves first: the first four passes need nothing else (requests complete in order)
 #pragma unroll
     for (int jr = 0; jr < R; jr++) w[jr][0] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr]);
+    if (T == 1) {
 #pragma unroll
-    for (int jr = 0; jr < R; jr++) w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
+        for (int jr = 0; jr < R; jr++) w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
+    }
     uint32_t warm0;      // loaded for its side effect only (the line ends up in L2)
     {
         const int lrow = (u_end - 1) / n_units, fi = lrow / row_tiles, frt = lrow % row_tiles;
@@ -412,30 +440,35 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
 
 size_t mx_lds_bytes() { return (size_t)2 * MX_ZBUF + (size_t)MX_WAVES * MX_STAGE + 2 * MX_WAVES * 16 * sizeof(float); }
 
-template <int R>
+template <int R, int T>
 int launch_mx(int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
     const size_t lds = mx_lds_bytes();
     static bs_lds_grant granted[BS_MAX_DEVICES];
-    const int st = bs_allow_lds((const void *)gemv_mx_kernel<R>, lds, granted);
+    const int st = bs_allow_lds((const void *)gemv_mx_kernel<R, T>, lds, granted);
     if (st != BS_OK) return st;
-    gemv_mx_kernel<R><<<grid, 64 * MX_WAVES, lds, s>>>(grp, x, N, K, n_units);
+    gemv_mx_kernel<R, T><<<grid, 64 * MX_WAVES, lds, s>>>(grp, x, N, K, n_units);
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
 
 }  // namespace
 
-// Shapes the block-scaled kernel runs: whole 512-column halves.
-bool bs_gemv_mx_takes(int N, int K, int R) {
-    if (N % 512 != 0 || K < 1 || K > 16) return false;
+// Shapes the block-scaled kernel runs: whole 512-column halves, one or two tokens.
+bool bs_gemv_mx_takes(int N, int K, int R, int T) {
+    if (N % 512 != 0 || K < 1 || K > 16 || T < 1 || T > 2) return false;
     return R == 1 || R == 2 || R == 4;
 }
 
-int bs_launch_gemv_mx(int R, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
-    if (!bs_gemv_mx_takes(N, K, R) || n_units != (int)bs_cdiv(N, MX_UNIT_COLS)) return BS_ERR_SHAPE;
+int bs_launch_gemv_mx(int R, int T, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s) {
+    if (!bs_gemv_mx_takes(N, K, R, T) || n_units != (int)bs_cdiv(N, MX_UNIT_COLS / T)) return BS_ERR_SHAPE;
+    if (T == 2) switch (R) {
+        case 1: return launch_mx<1, 2>(grid, grp, x, N, K, n_units, s);
+        case 2: return launch_mx<2, 2>(grid, grp, x, N, K, n_units, s);
+        default: return launch_mx<4, 2>(grid, grp, x, N, K, n_units, s);
+    }
     switch (R) {
-        case 1: return launch_mx<1>(grid, grp, x, N, K, n_units, s);
-        case 2: return launch_mx<2>(grid, grp, x, N, K, n_units, s);
-        default: return launch_mx<4>(grid, grp, x, N, K, n_units, s);
+        case 1: return launch_mx<1, 1>(grid, grp, x, N, K, n_units, s);
+        case 2: return launch_mx<2, 1>(grid, grp, x, N, K, n_units, s);
+        default: return launch_mx<4, 1>(grid, grp, x, N, K, n_units, s);
     }
 }

@@ -38,9 +38,9 @@ struct GemvGroup {
     int n;
 };
 
-// One-token decode on the block-scaled fp4 x fp6 MFMA (gemv_mx.hip).  Same unit order, partition,
-// partial layout and flush as gemv_kernel, but a unit spans MX_UNIT_COLS columns; rows per
+// One- and two-token decode on the block-scaled fp4 x fp6 MFMA (gemv_mx.hip).  Same unit order, partition,
+// partial layout and flush as gemv_kernel, but a unit spans MX_UNIT_COLS / T columns; rows per
 // workgroup = 8 waves x R x 16.
 constexpr int MX_UNIT_COLS = 1024;
-bool bs_gemv_mx_takes(int N, int K, int R);
-int bs_launch_gemv_mx(int R, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s);
+bool bs_gemv_mx_takes(int N, int K, int R, int T);
+int bs_launch_gemv_mx(int R, int T, int grid, const GemvGroup &grp, const half_t *x, int N, int K, int n_units, hipStream_t s);

@@ -143,18 +143,19 @@ int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles
 /*
  * Which decode kernel bs_forward runs for these dimensions: 0 none (strip kernel
  * or dense path), BS_DECODE_F16 the fp16-MFMA kernel (1..4 tokens per pass),
- * BS_DECODE_MX the block-scaled fp4 x fp6 MFMA kernel (one token; signs as the
- * fp4 operand, vt o x as three fp6 terms).  Negative = error status.
+ * BS_DECODE_MX the block-scaled fp4 x fp6 MFMA kernel (one or two tokens; signs
+ * as the fp4 operand, vt o x as three fp6 terms).  For more than four tokens the
+ * answer is that of the first pass.  Negative = error status.
  */
 #define BS_DECODE_F16 1
 #define BS_DECODE_MX  2
 int bs_decode_kernel(int I, int M, int N, int K, int T);
 
 /*
- * Test and benchmark hook: 0 = choose the one-token decode kernel by shape (the
- * default), BS_DECODE_F16 = always the fp16 kernel, BS_DECODE_MX = the
- * block-scaled kernel wherever it takes the shape (N % 512 == 0, x and its
- * operand images within LDS).  Process-wide and not synchronised: set it while
+ * Test and benchmark hook: 0 = choose the decode kernel of one- and two-token
+ * passes by shape (the default), BS_DECODE_F16 = always the fp16 kernel,
+ * BS_DECODE_MX = the block-scaled kernel wherever it takes the shape
+ * (N % 512 == 0, at most two tokens).  Process-wide and not synchronised: set it while
  * no other thread is inside the library.  Workspace sizes and bs_decode_plan
  * follow the setting.  No counterpart in the reference.
  */

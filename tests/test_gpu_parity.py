@@ -181,7 +181,7 @@ def decode_kernel():
     L.bs_set_decode_kernel(_lib.DECODE_AUTO)
 
 
-# one token through the block-scaled fp4 x fp6 kernel: every row-tile height (128 .. 1024 rows per workgroup),
+# one and two tokens through the block-scaled fp4 x fp6 kernel: every row-tile height (128 .. 1024 rows per workgroup),
 # ragged last row tiles, N a multiple of 512 but not of 1024 (a unit whose second half lies beyond N), ranks
 # below 16 (whole rank quads and a partial one missing), many blocks, several units per workgroup
 MX_CASES = [(1, 64, 512, 16), (1, 128, 1024, 16), (2, 256, 1536, 16), (4, 1024, 1024, 16), (3, 200, 1024, 5),
@@ -190,25 +190,26 @@ MX_CASES = [(1, 64, 512, 16), (1, 128, 1024, 16), (2, 256, 1536, 16), (4, 1024, 
             (48, 2500, 4096, 16), (200, 1100, 1536, 16), (16, 4096, 4096, 16), (5, 8192, 3584, 16)]
 
 
+@pytest.mark.parametrize("T", [1, 2])
 @pytest.mark.parametrize("I,M,N,K", MX_CASES)
-def test_forward_decode_block_scaled_kernel(I, M, N, K, decode_kernel):
+def test_forward_decode_block_scaled_kernel(I, M, N, K, T, decode_kernel):
     """The block-scaled kernel splits vt * x (fp16) into three fp6 terms per 32 columns, exact to under
     1e-4 of the block maximum: same tolerance as the fp16 kernel against float64, and the two kernels
     against each other."""
-    print(f"forward decode (block-scaled) I={I} M={M} N={N} K={K}", flush=True)
-    q, u, vt, x = synthetic_layer(M, N, I, 1, k=K, seed=I * 5 + K, signed_factors=(K != 16))
+    print(f"forward decode (block-scaled) I={I} M={M} N={N} K={K} T={T}", flush=True)
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=I * 5 + K + T, signed_factors=(K != 16))
     bias = (torch.randn(M, generator=torch.Generator().manual_seed(K)) * 0.01).half() if (I + K) % 2 else None
     exact, l0 = oracle_refs(q, u, vt, x, bias)
     args = (q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev()), None if bias is None else bias.to(dev()))
     decode_kernel(_lib.DECODE_MX)
-    assert _lib.lib().bs_decode_kernel(I, M, N, K, 1) == _lib.DECODE_MX
+    assert _lib.lib().bs_decode_kernel(I, M, N, K, T) == _lib.DECODE_MX
     y = IU.bitstack_forward_hip(*args)
     assert torch.equal(IU.bitstack_forward_hip(*args), y)                   # deterministic
     decode_kernel(_lib.DECODE_F16)
-    assert _lib.lib().bs_decode_kernel(I, M, N, K, 1) == _lib.DECODE_F16
+    assert _lib.lib().bs_decode_kernel(I, M, N, K, T) == _lib.DECODE_F16
     y16 = IU.bitstack_forward_hip(*args)
     y = y.cpu().numpy()
-    assert y.dtype == np.float16 and y.shape == (1, M)
+    assert y.dtype == np.float16 and y.shape == (T, M)
     assert_close(y, exact, "vs fp64")
     if I <= 16:
         assert_close(y, l0, "vs level-0 order")
@@ -218,7 +219,8 @@ def test_forward_decode_block_scaled_kernel(I, M, N, K, decode_kernel):
 def test_block_scaled_kernel_is_declined_where_it_does_not_apply(decode_kernel):
     decode_kernel(_lib.DECODE_MX)
     L = _lib.lib()
-    assert L.bs_decode_kernel(2, 256, 512, 16, 2) == _lib.DECODE_F16       # more than one token
+    assert L.bs_decode_kernel(2, 256, 512, 16, 2) == _lib.DECODE_MX        # two tokens: units of 512 columns
+    assert L.bs_decode_kernel(2, 256, 512, 16, 3) == _lib.DECODE_F16       # more than two tokens
     assert L.bs_decode_kernel(2, 256, 640, 16, 1) == 0                     # N not a multiple of 512: no decode kernel at all
     q, u, vt, x = synthetic_layer(256, 1024, 2, 3, seed=1)
     exact, _ = oracle_refs(q, u, vt, x)
