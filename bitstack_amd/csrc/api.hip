@@ -48,15 +48,18 @@ extern "C" int bs_set_dense_kernel(int mode) {
     return BS_OK;
 }
 
-extern "C" int64_t bs_workspace_bytes(int I, int M, int N, int K, int T) {
+// `library_ok`: the dense product may run on hipBLASLt (and then needs its scratch behind the weight)
+static int64_t workspace_need(int I, int M, int N, int K, int T, bool library_ok) {
     int st = forward_dims(I, M, N, K, T);
     if (st != BS_OK) return st;
     if (T == 0) return 0;
     int64_t gemv = bs_gemv_workspace_bytes(I, M, N, K, T);
     if (gemv > 0) return round_up(gemv, 256);
     // the rebuilt weight, then the library GEMM's own scratch where that is the kernel
-    return round_up((int64_t)M * N * 2, 256) + (dense_wants_library(M, N, T) ? BS_DENSE_LIBRARY_WORKSPACE : 0);
+    return round_up((int64_t)M * N * 2, 256) + (library_ok && dense_wants_library(M, N, T) ? BS_DENSE_LIBRARY_WORKSPACE : 0);
 }
+
+extern "C" int64_t bs_workspace_bytes(int I, int M, int N, int K, int T) { return workspace_need(I, M, N, K, T, true); }
 
 extern "C" int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave,
                               int *workgroups, int *partials_per_row) {
@@ -75,9 +78,9 @@ extern "C" int bs_decode_kernel(int I, int M, int N, int K, int T) {
 
 extern "C" int bs_set_decode_kernel(int mode) { return bs_gemv_set_kernel(mode); }
 
-extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void *x,
-                          const void *bias, void *y, int I, int M, int N, int K, int T,
-                          void *workspace, int64_t workspace_bytes, void *stream) {
+static int forward_impl(const uint8_t *packed, const void *u, const void *vt, const void *x,
+                        const void *bias, void *y, int I, int M, int N, int K, int T,
+                        void *workspace, int64_t workspace_bytes, void *stream, bool library_ok) {
     int st = forward_dims(I, M, N, K, T);
     if (st != BS_OK) return st;
     if (T == 0) return BS_OK;
@@ -85,7 +88,7 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     if (!bs_aligned(packed, 16) || !bs_aligned(vt, 16) || !bs_aligned(x, 16) || !bs_aligned(u, 8) ||
         !bs_aligned(y, 2) || !bs_aligned(bias, 2))
         return BS_ERR_ALIGN;
-    const int64_t need = bs_workspace_bytes(I, M, N, K, T);
+    const int64_t need = workspace_need(I, M, N, K, T, library_ok);
     if (need > 0 && (!workspace || workspace_bytes < need || !bs_aligned(workspace, 256)))
         return BS_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
@@ -99,12 +102,18 @@ extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, 
     half_t *w = (half_t *)workspace;
     st = bs_launch_reconstruct_packed(packed, (const half_t *)u, (const half_t *)vt, w, I, M, N, K, s);
     if (st != BS_OK) return st;
-    if (dense_wants_library(M, N, T)) {
+    if (library_ok && dense_wants_library(M, N, T)) {
         st = bs_launch_linear_library((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N,
                                       (char *)workspace + round_up((int64_t)M * N * 2, 256), s);
         if (st != BS_ERR_SHAPE) return st;      // enqueued, or failed for good; BS_ERR_SHAPE: not for this call
     }
     return bs_launch_linear_f16((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N, s);
+}
+
+extern "C" int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void *x,
+                          const void *bias, void *y, int I, int M, int N, int K, int T,
+                          void *workspace, int64_t workspace_bytes, void *stream) {
+    return forward_impl(packed, u, vt, x, bias, y, I, M, N, K, T, workspace, workspace_bytes, stream, true);
 }
 
 // ---- the forward for callers that cannot allocate ------------------------------------
@@ -137,15 +146,17 @@ extern "C" int bs_forward_static(const uint8_t *packed, const void *u, const voi
     int st = forward_dims(I, M, N, K, T);
     if (st != BS_OK) return st;
     if (T == 0) return BS_OK;
-    // sizes first: a call that would not fit is refused before any device is touched
-    const int64_t need = bs_workspace_bytes(I, M, N, K, T);
+    // sizes first: a call that would not fit is refused before any device is touched.  The dense product
+    // always runs this library's own kernel here: the vendor GEMM wants 64 MiB of scratch of its own, and
+    // setting it up allocates.
+    const int64_t need = workspace_need(I, M, N, K, T, false);
     if (need < 0) return (int)need;
     if (need > (int64_t)BS_STATIC_SCRATCH_BYTES) return BS_ERR_WORKSPACE;
     void *ws = nullptr;
     st = static_scratch(&ws);
     if (st != BS_OK) return st;
     // nothing in the scratch has to start at zero: every partial sum a call reads it has written before
-    return bs_forward(packed, u, vt, x, bias, y, I, M, N, K, T, ws, (int64_t)BS_STATIC_SCRATCH_BYTES, stream);
+    return forward_impl(packed, u, vt, x, bias, y, I, M, N, K, T, ws, (int64_t)BS_STATIC_SCRATCH_BYTES, stream, false);
 }
 
 // ---- grouped decode forward ---------------------------------------------------

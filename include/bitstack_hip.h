@@ -113,7 +113,8 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * hipMalloc).  No counterpart in the reference.  The scratch of the kernels is a
  * device array inside the library, BS_STATIC_SCRATCH_BYTES per GPU, held until
  * the process ends; the call allocates nothing and frees nothing.  Dimensions
- * whose bs_workspace_bytes exceeds BS_STATIC_SCRATCH_BYTES return
+ * whose scratch (bs_workspace_bytes, less the vendor GEMM's 64 MiB where
+ * bs_forward would use it) exceeds BS_STATIC_SCRATCH_BYTES return
  * BS_ERR_WORKSPACE: 64 MiB holds the partial sums of every 1..4-token forward of
  * the 8B and 70B linear shapes up to 36 blocks and of their 5..8-token forwards
  * up to 12 blocks; the strip kernel at several dozen tokens on the largest
@@ -121,7 +122,10 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * (more than 48 tokens, or N not a multiple of 128) need more and are refused.
  * All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (different streams, different host threads) race; calls on one
- * stream are ordered and safe.  Same results as bs_forward, bit for bit.
+ * stream are ordered and safe.  Same results as bs_forward, bit for bit; from
+ * 512 tokens on as bs_forward under bs_set_dense_kernel(BS_DENSE_OWN), because
+ * the dense product here always runs this library's own kernel (the vendor
+ * GEMM needs scratch of its own and allocates when it is set up).
  */
 #define BS_STATIC_SCRATCH_BYTES (64 << 20)
 int bs_forward_static(const uint8_t *packed, const void *u, const void *vt, const void *x,
