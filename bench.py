@@ -51,10 +51,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the T=4 and prefill side measurements")
-    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer", "scoring", "copy"], default=None,
+    ap.add_argument("--only", choices=["decode_8b", "decode_70b", "prefill", "one_layer", "scoring", "copy", "sweep_tokens"], default=None,
                     help="run just this side measurement and print its object (for profiling one path)")
     ap.add_argument("--batch", type=int, default=8, help="sequences decoded in lock step by --only decode_70b (1..48)")
     ap.add_argument("--prompt-len", type=int, default=2048, help="prompt tokens per sequence of --only decode_70b")
+    ap.add_argument("--tokens", type=int, default=2, help="tokens per forward of --only sweep_tokens (the 20-layer sweep at that count)")
     ap.add_argument("--layer", default="14336x4096x16x1",
                     help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
@@ -381,6 +382,18 @@ def main():
                                         "decode_plan": _lib.decode_plan(I, M, N, 16, T),
                                         "decode_kernel": {0: "none", 1: "gemv_kernel (fp16 MFMA)", 2: "gemv_mx_kernel (fp4 x fp6 MFMA)"}[
                                             lib.bs_decode_kernel(I, M, N, 16, T)]}}))
+        return
+    if a.only == "sweep_tokens":
+        # the 20-layer sweep at --tokens tokens per forward, events around every forward: the process to trace for
+        # the multi-token decode kernels
+        lt = build_sweep(a.tokens)
+        _, per = time_sweep(lt, max(3, a.steps // 2), 1, per_layer_events=True)
+        bt = sum(L.bytes for L in lt)
+        print(json.dumps({"sweep_tokens": {"tokens": a.tokens, "us_per_pass": round(sum(per) * 1e3, 1),
+                                           "GBps": round(bt / (sum(per) * 1e-3) / 1e9, 1),
+                                           "layers": [{"M": L.M, "N": L.N, "I": L.I, "us": round(ms * 1e3, 2),
+                                                       "kernel": int(lib.bs_decode_kernel(L.I, L.M, L.N, 16, L.T))}
+                                                      for L, ms in zip(lt, per)]}}))
         return
     if a.only == "copy":
         # a plain device-to-device copy of 256 MiB, five times: what the FETCH_SIZE / WRITE_SIZE counters read for a
