@@ -32,6 +32,15 @@ def assert_close(got, ref, what, max_rel=MAX_REL, mean_rel=MEAN_REL):
     assert mx <= max_rel and mn <= mean_rel, f"{what}: max_rel={mx:.3e} mean_rel={mn:.3e}"
 
 
+@pytest.fixture(params=[_lib.DECODE_AUTO, _lib.DECODE_MX], ids=["planned_kernel", "block_scaled_kernel"])
+def decode_kernel_mode(request):
+    """The grouped launches once as planned and once with the block-scaled kernel on every one- and two-token
+    pass that it takes (so that small groups reach it too)."""
+    assert _lib.lib().bs_set_decode_kernel(request.param) == 0
+    yield request.param
+    assert _lib.lib().bs_set_decode_kernel(_lib.DECODE_AUTO) == 0
+
+
 def make_group(shapes, N, T, seed, bias=False):
     """shapes: [(I, M)]; returns (MatrixGroup on the GPU, x on the CPU, fp64 reference outputs per matrix)."""
     mats, refs, x = [], [], None
@@ -53,7 +62,7 @@ GROUP_CASES = [([(3, 512), (5, 128), (2, 128)], 512, 1), ([(3, 4096), (5, 1024),
 
 
 @pytest.mark.parametrize("shapes,N,T", GROUP_CASES)
-def test_group_forward_side_by_side(shapes, N, T):
+def test_group_forward_side_by_side(shapes, N, T, decode_kernel_mode):
     print(f"group forward {shapes} N={N} T={T}", flush=True)
     grp, x, refs = make_group(shapes, N, T, seed=11, bias=(T % 2 == 0))
     y = IU.bitstack_forward_group_hip(grp, x.to(dev())).cpu().numpy()
@@ -68,7 +77,7 @@ def test_group_forward_side_by_side(shapes, N, T):
 
 
 @pytest.mark.parametrize("I,M,N,T", [(3, 512, 1024, 1), (2, 4096, 4096, 1), (2, 256, 512, 6), (2, 300, 640, 12)])
-def test_group_forward_residual(I, M, N, T):
+def test_group_forward_residual(I, M, N, T, decode_kernel_mode):
     print(f"group residual I={I} M={M} N={N} T={T}", flush=True)
     grp, x, refs = make_group([(I, M)], N, T, seed=21)
     res = (torch.randn(T, M, generator=torch.Generator().manual_seed(2)) * 0.1).half()
@@ -79,7 +88,7 @@ def test_group_forward_residual(I, M, N, T):
 
 
 @pytest.mark.parametrize("I0,I1,M,N,T", [(3, 2, 1024, 512, 1), (2, 4, 14336, 4096, 1), (2, 2, 512, 1024, 7), (2, 3, 1024, 2048, 24)])
-def test_group_forward_swiglu(I0, I1, M, N, T):
+def test_group_forward_swiglu(I0, I1, M, N, T, decode_kernel_mode):
     print(f"group swiglu I={I0},{I1} M={M} N={N} T={T}", flush=True)
     grp, x, refs = make_group([(I0, M), (I1, M)], N, T, seed=31)
     # scale so that the gate spans the non-linear range of silu
@@ -348,7 +357,7 @@ def test_decoder_round_trips_through_a_checkpoint(tmp_path):
                                               ([(2, 512), (3, 128)], 1024, 40, "none"),
                                               ([(2, 256), (2, 256)], 512, 48, "swiglu"),
                                               ([(2, 300)], 1536, 3, "none")])
-def test_group_forward_with_input_rms(shapes, N, T, mode):
+def test_group_forward_with_input_rms(shapes, N, T, mode, decode_kernel_mode):
     """bs_forward_group_rms: the RMSNorm in front of the matrices without a launch of its own.  The
     caller folds the norm weight into vt; the launch scales by rsqrt(mean(x^2) + eps)."""
     print(f"group rms {shapes} N={N} T={T} {mode}", flush=True)
