@@ -42,6 +42,8 @@ PEAK_CLOCK_HZ = 2.4e9         # MI355X peak engine clock
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 BLOCKS = [1, 2, 4, 8, 16]
 PREFILL_T = [16, 128, 512, 2048]
+PREFILL_WARM_MS = 60.0      # untimed load in front of every prefill timing (clock recovery after a pause)
+SIDE_WARM_MS = 30.0         # the same in front of the 2-, 4- and 16-token side measurements
 
 
 def parse():
@@ -300,13 +302,21 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
-    def time_fns(fns, steps, warmup, per_layer_events):
+    def time_fns(fns, steps, warmup, per_layer_events, warm_ms=0.0):
         """The callables in turn, `steps` passes after `warmup` untimed ones: wall clock of the timed
-        passes and, with events around every call, the mean time of each callable (ms)."""
+        passes and, with events around every call, the mean time of each callable (ms).  `warm_ms`: keep
+        running untimed passes until that much wall time has passed (after a pause the shader clock needs
+        tens of milliseconds of load to come back: a variant timed first would otherwise look 10-20 % slower
+        than the same kernels timed later)."""
         for _ in range(warmup):
             for f in fns:
                 f()
         torch.cuda.synchronize()
+        t_warm = time.perf_counter()
+        while (time.perf_counter() - t_warm) * 1e3 < warm_ms:
+            for f in fns:
+                f()
+            torch.cuda.synchronize()
         ev = None
         if per_layer_events:
             ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
@@ -327,15 +337,15 @@ def main():
                          for j in range(len(fns))]          # ms per forward
         return wall, per_layer
 
-    def time_sweep(layers, steps, warmup, per_layer_events):
+    def time_sweep(layers, steps, warmup, per_layer_events, warm_ms=0.0):
         ws = workspace_for(layers)
-        return time_fns([make_forward(L, lib, ws, stream) for L in layers], steps, warmup, per_layer_events)
+        return time_fns([make_forward(L, lib, ws, stream) for L in layers], steps, warmup, per_layer_events, warm_ms)
 
     def prefill_side(detail):
         pre = {}
         for T in PREFILL_T:
             lp = build_sweep(T, blocks=[8])
-            _, perp = time_sweep(lp, 3, 1, per_layer_events=True)
+            _, perp = time_sweep(lp, 3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
             useful = sum(2.0 * L.M * L.N * L.T + 2.0 * 16 * L.I * L.M * L.N for L in lp)
             tp = sum(perp) * 1e-3
             pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
@@ -348,12 +358,15 @@ def main():
                 import torch.nn.functional as F
                 from bitstack_amd.utils.inference_utils import unpack_and_reconstruct_w_hip
                 lib.bs_set_dense_kernel(_lib.DENSE_OWN)
-                _, own = time_sweep(lp, 3, 1, per_layer_events=True)
+                _, own = time_sweep(lp, 3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
                 lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
                 pre[f"T{T}"]["own_dense_kernel_useful_tflops"] = round(useful / (sum(own) * 1e-3) / 1e12, 1)
                 _, lvl3 = time_fns([(lambda L=L: F.linear(L.x, unpack_and_reconstruct_w_hip(L.q, L.u, L.vt))) for L in lp],
-                                   3, 1, per_layer_events=True)
+                                   3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
                 pre[f"T{T}"]["level3_rebuild_plus_torch_linear_useful_tflops"] = round(useful / (sum(lvl3) * 1e-3) / 1e12, 1)
+                pre[f"T{T}"]["us_per_layer"] = {"layers": [f"{L.M}x{L.N}" for L in lp], "default": [round(v * 1e3, 1) for v in perp],
+                                                "own_dense_kernel": [round(v * 1e3, 1) for v in own],
+                                                "level3": [round(v * 1e3, 1) for v in lvl3]}
             detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
                         "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
                        for L, ms in zip(lp, perp)]
@@ -387,7 +400,7 @@ def main():
         # the 20-layer sweep at --tokens tokens per forward, events around every forward: the process to trace for
         # the multi-token decode kernels
         lt = build_sweep(a.tokens)
-        _, per = time_sweep(lt, max(3, a.steps // 2), 1, per_layer_events=True)
+        _, per = time_sweep(lt, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
         bt = sum(L.bytes for L in lt)
         print(json.dumps({"sweep_tokens": {"tokens": a.tokens, "us_per_pass": round(sum(per) * 1e3, 1),
                                            "GBps": round(bt / (sum(per) * 1e-3) / 1e9, 1),
@@ -522,11 +535,11 @@ def main():
     if not a.no_extras:
         # ------------------------------------------------------------ T = 2 sweep (block-scaled kernel, 512-column units)
         l2 = build_sweep(2)
-        _, per2 = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True)
+        _, per2 = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
         b2 = sum(L.bytes for L in l2)
         t2 = sum(per2) * 1e-3
         lib.bs_set_decode_kernel(_lib.DECODE_F16)
-        _, per2f = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True)
+        _, per2f = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
         lib.bs_set_decode_kernel(_lib.DECODE_AUTO)
         out["t2"] = {"GBps": round(b2 / t2 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b2 / t2 / 1e9 / HBM_PEAK_GBS, 2),
                      "GBps_fp16_kernel_forced": round(b2 / (sum(per2f) * 1e-3) / 1e9, 1)}
@@ -535,7 +548,7 @@ def main():
         del l2
         # ------------------------------------------------------------ T = 4 sweep (MFMA-bound side)
         l4 = build_sweep(4)
-        _, per4 = time_sweep(l4, max(3, a.steps // 2), 1, per_layer_events=True)
+        _, per4 = time_sweep(l4, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
         b4 = sum(L.bytes for L in l4)
         flops4 = sum(2.0 * 16 * L.I * L.M * L.N * L.T for L in l4)
         t4 = sum(per4) * 1e-3
@@ -546,7 +559,7 @@ def main():
         del l4
         # ------------------------------------------------------------ T = 16 sweep (strip kernel: batched decode)
         l16 = build_sweep(16)
-        _, per16 = time_sweep(l16, max(3, a.steps // 2), 1, per_layer_events=True)
+        _, per16 = time_sweep(l16, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
         b16 = sum(L.bytes for L in l16)
         t16 = sum(per16) * 1e-3
         out["t16"] = {"GBps": round(b16 / t16 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b16 / t16 / 1e9 / HBM_PEAK_GBS, 2),
