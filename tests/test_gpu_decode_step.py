@@ -229,6 +229,36 @@ def dense_weights(model):
     return w
 
 
+@pytest.mark.parametrize("batch", [1, 2, 4])
+def test_fused_step_at_8b_layer_widths_matches_float64_decoder(batch):
+    """One decoder layer at the real Llama-3.1-8B widths (hidden 4096, intermediate 14336, 32 query / 8 KV heads), one,
+    two and four sequences: the grouped launches then run on the kernels the full model runs on (q/k/v and gate/up with the RMS
+    scale and SwiGLU on the block-scaled kernel at one and two tokens and on the fp16 kernel at four, the residual epilogues), against the float64 decoder
+    on the float64-rebuilt weights."""
+    shape = LlamaShape(layers=1, hidden=4096, intermediate=14336, heads=32, kv_heads=8, vocab=512)
+    cfg = {f"layer.0.{p}": b for p, b in zip(PROJ, (3, 2, 4, 3, 2, 3, 2))}
+    max_len = 16
+    m = SyntheticLlamaDecoder(shape, cfg, max_len, dev(), seed=8, batch=batch)
+    with torch.no_grad():
+        g = torch.Generator(device=dev()).manual_seed(3)
+        m.norm_w.copy_(1 + 0.2 * torch.randn(m.norm_w.shape, device=dev(), generator=g))
+        m.embed.mul_(30.0)
+    # the gate/up and q/k/v groups are large enough for the block-scaled kernel, at two tokens too
+    gu = [(cfg["layer.0.mlp.gate_proj"], 14336), (cfg["layer.0.mlp.up_proj"], 14336)]
+    assert _lib.lib().bs_decode_kernel(gu[0][0] + gu[1][0], 14336, 4096, 16, batch) == (_lib.DECODE_MX if batch <= 2 else _lib.DECODE_F16)
+    w = dense_weights(m)
+    orcs = [LO.LlamaOracle(w, shape.layers, shape.heads, shape.kv_heads, shape.head_dim, shape.rope_theta, shape.rms_eps, max_len)
+            for _ in range(batch)]
+    tokens = torch.randint(0, shape.vocab, (batch, 5), generator=torch.Generator().manual_seed(2))
+    for j in range(tokens.shape[1]):
+        m.token.copy_(tokens[:, j])
+        m.step_fused()
+        got = m.logits.float().cpu().numpy()
+        for s in range(batch):
+            want = orcs[s].step(int(tokens[s, j]))
+            assert_close(got[s], want, f"8B widths, fused vs float64, position {j} seq {s}", 2e-2, 4e-3)
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 def test_fused_step_matches_torch_step_and_float64_decoder(batch):
     print(f"fused decode step batch={batch}", flush=True)
