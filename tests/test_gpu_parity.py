@@ -648,3 +648,53 @@ def test_forward_with_2_31_weights_takes_the_rebuild_path():
     tail = C.reconstruct_w(qs[:, -N // 8:].copy(), u[:, M - 1:].cpu().numpy(), vt.cpu().numpy())
     got = w[M - 1:].cpu().numpy()
     assert np.all(np.abs(got.astype(np.float64) - tail.astype(np.float64)) <= np.spacing(np.abs(tail)).astype(np.float64))
+
+
+# ------------------------------------------------------------- seeded random shapes, every kernel choice forced
+def _random_forced_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        kind = rng.integers(0, 5)
+        if kind == 0:      # decode kernels, many blocks (long partial-sum lists)
+            N = 512 * int(rng.integers(1, 9)); M = int(rng.integers(1, 3000)); T = int(rng.integers(1, 5)); I = int(rng.integers(1, 40))
+        elif kind == 1:    # one and two tokens on wide matrices (several units per workgroup)
+            N = 512 * int(rng.integers(1, 17)); M = 64 * int(rng.integers(1, 120)); T = int(rng.integers(1, 3)); I = int(rng.integers(1, 20))
+        elif kind == 2:    # strip kernel
+            N = 128 * int(rng.integers(1, 40)); M = int(rng.integers(1, 2500)); T = int(rng.integers(5, 49)); I = int(rng.integers(1, 12))
+        elif kind == 3:    # rebuild + dense, ragged everything
+            N = 8 * int(rng.integers(1, 300)); M = int(rng.integers(1, 1500)); T = int(rng.integers(1, 700)); I = int(rng.integers(1, 6))
+        else:              # either side of the token count where the vendor GEMM takes over
+            N = 1024 * int(rng.integers(1, 5)); M = 512 * int(rng.integers(1, 9)); T = int(rng.choice([1, 2, 511, 512, 600, 1024])); I = int(rng.integers(1, 10))
+        cases.append((I, M, N, T, int(rng.choice([16, 16, 16, 12, 5, 1])), int(rng.integers(0, 3)), int(rng.integers(0, 3))))
+    return cases
+
+
+@pytest.mark.parametrize("I,M,N,T,K,decode_mode,dense_mode", _random_forced_cases(72, 20250309))
+def test_forward_random_shapes_forced_kernels(I, M, N, T, K, decode_mode, dense_mode, decode_kernel):
+    """bs_forward with the decode kernel (planned / fp16 / block-scaled) and the dense kernel (planned / own /
+    hipBLASLt) forced at random, against a float64 evaluation of the closed form on the GPU (signs through
+    the bit-exact unpack kernel): deterministic, and within the stated tolerance whatever runs the shape."""
+    print(f"forward random forced I={I} M={M} N={N} T={T} K={K} decode={decode_mode} dense={dense_mode}", flush=True)
+    from bitstack_amd.utils import pack_utils as PU
+    g = torch.Generator(device=dev()).manual_seed(I * 7 + M + N + T)
+    q = torch.randint(0, 256, (I, (M * N + 7) // 8), dtype=torch.uint8, device=dev(), generator=g)
+    sc = (0.02 / torch.arange(1, I + 1, device=dev()).float()).view(I, 1, 1)
+    u = (torch.randn(I, M, K, device=dev(), generator=g) * sc).half()
+    vt = (torch.randn(I, K, N, device=dev(), generator=g) * sc.sqrt()).half()
+    x = torch.randn(T, N, device=dev(), generator=g).half()
+    bias = (torch.randn(M, device=dev(), generator=g) * 0.01).half() if (M + T) % 3 == 0 else None
+    decode_kernel(decode_mode)
+    assert _lib.lib().bs_set_dense_kernel(dense_mode) == 0
+    try:
+        y = IU.bitstack_forward_hip(q, u, vt, x, bias)
+        assert torch.equal(IU.bitstack_forward_hip(q, u, vt, x, bias), y)
+    finally:
+        _lib.lib().bs_set_dense_kernel(_lib.DENSE_AUTO)
+    w = torch.zeros(M, N, device=dev(), dtype=torch.float64)
+    for i in range(I):
+        w += PU.unpack_sign(q[i], (M, N)).double() * (u[i].double() @ vt[i].double())
+    want = x.double() @ w.T
+    if bias is not None:
+        want = want + bias.double()
+    assert_close(y.cpu().numpy(), want.cpu().numpy(), "vs float64 on the GPU")
