@@ -22,7 +22,7 @@ Extra objects on the same JSON line:
   cpu_baseline  the reference's CPU path (level 0) restated in torch-CPU ops,
                 timed on this host on one pass of the same sweep.
   t2, t4, t16, prefill   the same sweep at 2, 4 and 16 tokens, and the prefill configuration
-                (I = 8, T in {16, 128, 512, 2048}) as useful TFLOP/s.
+                (I = 8, T in {16, 64, 128, 512, 2048}) as useful TFLOP/s.
   decode_8b     tokens/s of a random-init Llama-3.1-8B-shape decode loop built
                 around the same forward (batch 1, 256 greedy tokens).
 """
@@ -41,7 +41,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 PEAK_CLOCK_HZ = 2.4e9         # MI355X peak engine clock
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 BLOCKS = [1, 2, 4, 8, 16]
-PREFILL_T = [16, 128, 512, 2048]
+PREFILL_T = [16, 64, 128, 512, 2048]
 PREFILL_WARM_MS = 60.0      # untimed load in front of every prefill timing (clock recovery after a pause)
 SIDE_WARM_MS = 30.0         # the same in front of the 2-, 4- and 16-token side measurements
 

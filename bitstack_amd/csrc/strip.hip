@@ -258,6 +258,227 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
     }
 }
 
+// ---- 49 to 96 tokens: the same patches, the strips walked by the workgroup -----------------------
+// With more token tiles the partial sums of strip_forward_kernel ([strip group, T, M] floats) outgrow the
+// weight itself, so here a workgroup keeps y[T, its 128 rows] in registers (TT accumulators per wave) and
+// walks a run of strips: per chunk of `sg` strips it stages the x and vt slices in LDS (one barrier before,
+// one after), every wave rebuilds its 16 rows of those strips patch by patch and multiplies them into the
+// accumulators at once.  The weight never exists outside registers, and scratch holds one partial per
+// COLUMN GROUP (a handful), not per strip.  The columns are cut into as many groups as it takes to fill the
+// chip with workgroups of 128 rows; workgroups of one column group sit on one XCD and share its vt slices.
+struct WideMat {
+    const uint8_t *packed;
+    const half_t *u, *vt;
+    float *part;
+    int I, M, sg, n_chunk, row_tiles;
+};
+
+template <int TT>
+__global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, const half_t *__restrict__ x, int N, int K, int T) {
+    constexpr int WAVES = 8, NT = 64 * WAVES, RS = 16 * WAVES;
+    extern __shared__ __attribute__((aligned(16))) half_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lm = lane & 15, g = lane >> 4;
+    int cgroup, rt;
+    {
+        const int nb = gridDim.x, xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+        const int base = nb >> 3, rem = nb & 7;
+        const int v = xcd * base + min(xcd, rem) + loc;
+        cgroup = v / mat.row_tiles;
+        rt = v - cgroup * mat.row_tiles;
+    }
+    const uint8_t *__restrict__ packed = mat.packed;
+    const half_t *__restrict__ u = mat.u;
+    const half_t *__restrict__ vt = mat.vt;
+    const int I = mat.I, M = mat.M, sg = mat.sg, n_chunk = mat.n_chunk;
+    const int xstride = sg * SF_COLS + 8;           // halves per token row of the x image
+    half_t *xl = lds;                               // [TT * 16][xstride]
+    half_t *vl = lds + TT * 16 * xstride;           // [sg][I][VBLOCK]
+    const int strips = N / SF_COLS;
+    const int first_strip = cgroup * n_chunk * sg;  // this workgroup's strips: first_strip .. + n_chunk * sg - 1, those below `strips`
+    const int64_t row_bytes = N >> 3;
+    const int64_t block_bytes = (int64_t)M * row_bytes;
+
+    const int sr = tid & 15, sp = (tid >> 4) & 15;  // staging role: rank, piece of 8 columns
+    const int spair = tid >> 8;                     // ... and which of the two (strip, block) pairs staged side by side
+    const int sh_byte = 24 - 8 * g;                 // brings the lane's byte of a sign word to the top
+    const int acol = 8 * (lm >> 2) + (lm & 3);
+    const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
+
+    const int m0 = rt * RS + wave * 16;
+    const int row = min(m0 + lm, M - 1);
+    const uint32_t off_u = (uint32_t)(row * K + 4 * g) * 2u;              // bytes: this lane's u row (its four ranks) and sign row
+    const uint32_t off_s = (uint32_t)row * (uint32_t)row_bytes;
+    auto load_block = [&](int i, int strip, half4_t &b, uint4_t &sw) {
+        const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
+        const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
+        if (K == 16) {
+            b = *reinterpret_cast<const half4_t *>(up);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
+        }
+        const uint8_t *sb = packed + i * block_bytes + ((strip * SF_COLS) >> 3);
+        sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
+    };
+    // The (strip, block) pairs of this wave form one sequence over all its chunks; the sign and u loads run two
+    // pairs ahead, unconditionally (behind the last strip they repeat it).
+    half4_t b_cur, b_n1, b_n2;
+    uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+    int pf_i = 0, pf_strip = first_strip;
+    auto request = [&](half4_t &b, uint4_t &sw) {
+        load_block(pf_i, min(pf_strip, strips - 1), b, sw);
+        if (++pf_i == I) {
+            pf_i = 0;
+            pf_strip++;
+        }
+    };
+    request(b_cur, sw_cur);
+    request(b_n1, sw_n1);
+
+    float4_t yacc[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    const half_t *xfrag = xl + lm * xstride + 8 * g;   // token lm of a tile, columns 32 (s / 2) + 8 g + 4 (s % 2) .. + 3 of patch s
+
+    for (int ch = 0; ch < n_chunk; ch++) {
+        const int s_begin = first_strip + ch * sg;
+        const int ns = max(0, min(sg, strips - s_begin));       // the same for every thread of the workgroup
+        const int n0 = s_begin * SF_COLS;
+        if (ch > 0) __syncthreads();                // everybody has finished with the previous images
+        // x image: token rows beyond T are zero
+        for (int idx = tid; idx < TT * 16 * ns * 16; idx += NT) {
+            const int t = idx / (ns * 16), piece = idx % (ns * 16);
+            half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (t < T) v = *reinterpret_cast<const half8_t *>(x + (int64_t)t * N + n0 + 8 * piece);
+            *reinterpret_cast<half8_t *>(xl + t * xstride + 8 * piece) = v;
+        }
+        // vt slices, four (strip, block) pairs per thread at a time so that their loads are in flight together
+        for (int q0 = 0; q0 < ns * I; q0 += 8) {
+            half8_t v[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int qi = min(q0 + k * 2 + spair, ns * I - 1), q = qi / I, i = qi - q * I;
+                v[k] = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
+                if (sr < K) v[k] = *reinterpret_cast<const half8_t *>(vt + ((int64_t)i * K + sr) * N + n0 + q * SF_COLS + 8 * sp);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                if (q0 + k * 2 + spair < ns * I) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vl[(q0 + k * 2 + spair) * VBLOCK + (8 * sp + e) * VSTRIDE + sp * VGROUP_PAD + sr] = v[k][e];
+                }
+            }
+        }
+        __syncthreads();
+
+        for (int q = 0; q < ns; q++) {
+            float4_t acc[8];
+#pragma unroll
+            for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < I; i++) {
+                request(b_n2, sw_n2);
+                const uint4_t swc = sw_cur;         // bit 1 means +1: the product enters negated, times -1.0f
+                const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
+                half4_t a[8];
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
+                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                for (int s = 0; s < 8; s++) {
+                    const float4_t p = p_next;
+                    if (s + 1 < 8)
+                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
+                        acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
+                    }
+                }
+                b_cur = b_n1;
+                sw_cur = sw_n1;
+                b_n1 = b_n2;
+                sw_n1 = sw_n2;
+            }
+            // y[token, row] += x[token, these columns] . w[row, these columns], w rounded to fp16 as the dense path rounds it
+            const half_t *xq = xfrag + q * SF_COLS;
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) {
+                    const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
+                    yacc[tt] = __builtin_amdgcn_mfma_f32_16x16x16f16(xf, wf, yacc[tt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (m0 + lm < M) {
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int t = 16 * tt + 4 * g + v;
+                if (t < T) mat.part[((int64_t)cgroup * T + t) * M + m0 + lm] = yacc[tt][v];
+            }
+    }
+}
+
+// Column groups and strips per chunk of the walked kernel: two workgroups per CU (LDS), about two per CU in all.
+struct WidePlan {
+    int tt, sg, n_chunk, col_groups, row_tiles;
+    size_t lds;
+    bool worth;      // expected to beat rebuild + dense kernel
+};
+// Up to six token tiles two workgroups share a CU (118-125 registers); seven and eight tiles take 133 and 159, one
+// workgroup per CU, and lose to rebuild + dense kernel on every large shape.
+constexpr int WIDE_MIN_T = 49, WIDE_MAX_T = 96;
+
+WidePlan make_wide_plan(int I, int M, int N, int T) {
+    WidePlan p;
+    p.tt = (T + 15) / 16;
+    p.row_tiles = (int)bs_cdiv(M, 128);
+    const int strips = N / SF_COLS;
+    p.sg = 0;
+    for (int sg = 8; sg >= 1; sg >>= 1) {
+        const size_t lds = ((size_t)sg * I * VBLOCK + (size_t)p.tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
+        if (lds * 2 <= 160 * 1024 || sg == 1) {
+            p.sg = sg;
+            p.lds = lds;
+            break;
+        }
+    }
+    const int chunks = (int)bs_cdiv(strips, p.sg);
+    // as many column groups as fill the workgroup slots of the chip (two per CU) without a second round
+    const int slots = 512;
+    int cg = slots / p.row_tiles;
+    if (cg > chunks) cg = chunks;
+    if (cg < 1) cg = 1;
+    p.n_chunk = (int)bs_cdiv(chunks, cg);
+    p.col_groups = (int)bs_cdiv(chunks, p.n_chunk);
+    // Measured against rebuild + dense kernel (8B layer shapes, layers alternating): per block both cost about the
+    // same, but the walked kernel saves the round trip of the weight through memory (37 against 49-78 us of fixed
+    // cost on the large shapes), so it wins - by 1.2-1.7x - wherever its workgroups fill the chip, and with few
+    // blocks and up to 80 tokens also where they do not (14336 rows: 448 workgroups for 512 slots).
+    const int grid = p.row_tiles * p.col_groups;
+    // (up to one workgroup per CU nothing is uneven; beyond, the busiest CU holds a whole number of rounds of two)
+    const double fill = grid <= slots / 2 ? 1.0 : (double)grid / (double)(bs_cdiv(grid, slots) * slots);
+    p.worth = fill >= 0.95 || (I <= 6 && p.tt <= 5);
+    return p;
+}
+
+template <int TT>
+int launch_wide(const WideMat &m, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
+    static bs_lds_grant granted[BS_MAX_DEVICES];
+    const int st = bs_allow_lds((const void *)strip_wide_kernel<TT>, lds, granted);
+    if (st != BS_OK) return st;
+    strip_wide_kernel<TT><<<grid, 512, lds, s>>>(m, x, N, K, T);
+    BS_LAUNCH_CHECK();
+    return BS_OK;
+}
+
 struct StripPlan {
     int tt, sg, groups, gx, row_groups, rows_per_wg;
     size_t lds;
@@ -330,8 +551,14 @@ int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int 
 // Partial sums per output (groups of strips) when this path takes the shape, else 0.
 int bs_strip_partials(int I, int M, int N, int K, int T) {
     (void)K;
-    if (I < 1 || M < 1 || T < 1 || T > 48 || N % SF_COLS != 0) return 0;
+    if (I < 1 || M < 1 || T < 1 || T > WIDE_MAX_T || N % SF_COLS != 0) return 0;
     if ((int64_t)M * N >= ((int64_t)1 << 34)) return 0;
+    if (T >= WIDE_MIN_T) {
+        // the walked kernel: 32-bit row offsets, and an LDS image of one strip that leaves room for two workgroups
+        if ((int64_t)M * (N >> 3) >= ((int64_t)1 << 32) || (int64_t)M * K * 2 >= ((int64_t)1 << 32)) return 0;
+        const WidePlan p = make_wide_plan(I, M, N, T);
+        return (p.lds * 2 <= 160 * 1024 && p.worth && p.col_groups <= 1024) ? p.col_groups : 0;
+    }
     if (strip_lds(I, token_tiles(T), 1) > 160 * 1024) return 0;
     const StripPlan p = make_strip_plan(I, M, N, T);
     return p.groups <= 1024 ? p.groups : 0;
@@ -343,6 +570,19 @@ int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *con
                           const int *I, const int *M, float *const *part, float *ssq, const half_t *x,
                           int N, int K, int T, hipStream_t s) {
     if (n < 1 || n > STRIP_MAX_GROUP || !bs_aligned(x, 16)) return BS_ERR_SHAPE;
+    if (T >= WIDE_MIN_T) {
+        // one matrix, no sums of squares: the walked kernel serves bs_forward's 49..128-token calls only
+        if (n != 1 || ssq || bs_strip_partials(I[0], M[0], N, K, T) == 0) return BS_ERR_SHAPE;
+        if (!bs_aligned(packed[0], 16) || !bs_aligned(vt[0], 16) || !bs_aligned(u[0], 8)) return BS_ERR_SHAPE;
+        const WidePlan p = make_wide_plan(I[0], M[0], N, T);
+        const WideMat m{packed[0], u[0], vt[0], part[0], I[0], M[0], p.sg, p.n_chunk, p.row_tiles};
+        const int grid = p.row_tiles * p.col_groups;
+        switch (p.tt) {
+            case 4: return launch_wide<4>(m, grid, p.lds, x, N, K, T, s);
+            case 5: return launch_wide<5>(m, grid, p.lds, x, N, K, T, s);
+            default: return launch_wide<6>(m, grid, p.lds, x, N, K, T, s);
+        }
+    }
     StripGroup grp;
     grp.n = n;
     grp.ssq = ssq;

@@ -97,7 +97,10 @@ int64_t bs_workspace_bytes(int I, int M, int N, int K, int T);
  * vt_i o x, scaled by u_i, all blocks in one pass; N % 512 == 0); 5 <= T <= 48
  * the strip kernel (16 x 16 patches of the weight rebuilt in registers and
  * multiplied by x at once, the weight never stored; N % 128 == 0; when it does
- * not take the shape, T <= 8 is two GEMV passes); larger T rebuilds the
+ * not take the shape, T <= 8 is two GEMV passes); 49 <= T <= 96 the same
+ * patches with the strips walked by workgroups of 128 rows, where that beats
+ * the next path (N % 128 == 0, vt of all blocks of a strip within 40 KB of
+ * LDS, workgroups that fill the chip or at most 6 blocks); larger T rebuilds the
  * weight once into `workspace` and runs a dense MFMA GEMM.  Requires
  * N % 8 == 0.  `workspace` must hold bs_workspace_bytes(...) bytes, 256-byte
  * aligned; its contents on entry do not matter and it may be reused by the
@@ -119,7 +122,7 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * the 8B and 70B linear shapes up to 36 blocks and of their 5..8-token forwards
  * up to 12 blocks; the strip kernel at several dozen tokens on the largest
  * matrices and every forward that rebuilds a weight of more than 32 Mi elements
- * (more than 48 tokens, or N not a multiple of 128) need more and are refused.
+ * (more than 96 tokens, or N not a multiple of 128) need more and are refused.
  * All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (different streams, different host threads) race; calls on one
  * stream are ordered and safe.  Same results as bs_forward, bit for bit; from

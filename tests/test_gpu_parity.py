@@ -279,6 +279,51 @@ STRIP_CASES = [(1, 16, 128, 5, 16), (3, 100, 384, 9, 16), (2, 65, 1152, 17, 7), 
                (3, 1000, 1024, 33, 16), (2, 4096, 4096, 48, 16), (4, 333, 640, 41, 5)]
 
 
+# 49..96 tokens: the same patches with the strips walked by a workgroup of 128 rows (4-6 token tiles): ragged rows and
+# token tiles, ranks below 16, one strip and several per chunk (few blocks leave room in LDS), several chunks per
+# workgroup, row counts whose workgroups do not fill the chip (few blocks: still taken), one column group and many
+WIDE_CASES = [(2, 128, 128, 49, 16), (3, 1000, 1152, 64, 16), (1, 4096, 4096, 96, 16), (8, 4096, 4096, 65, 16),
+              (3, 14336, 4096, 80, 16), (2, 4096, 14336, 50, 16), (5, 333, 640, 77, 5), (12, 1024, 4096, 96, 16),
+              (4, 130, 2432, 81, 12), (6, 2000, 1024, 49, 1)]
+
+
+@pytest.mark.parametrize("I,M,N,T,K", WIDE_CASES)
+def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K):
+    print(f"forward walked strips I={I} M={M} N={N} T={T} K={K}", flush=True)
+    L = _lib.lib()
+    # the path is taken: the scratch is g x ([T, M] partial sums + T sums of squares) for g column groups, not the weight
+    need = int(L.bs_workspace_bytes(I, M, N, K, T))
+    groups = need // (T * (M + 1) * 4)
+    assert groups >= 1 and need == (groups * T * (M + 1) * 4 + 255) // 256 * 256 and need != M * N * 2
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=5 * I + T, signed_factors=True)
+    bias = (torch.randn(M, generator=torch.Generator().manual_seed(T)) * 0.05).half() if T % 2 else None
+    exact, l0 = oracle_refs(q, u, vt, x, bias)
+    qd, ud, vd, xd = q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())
+    bd = None if bias is None else bias.to(dev())
+    y = IU.bitstack_forward_hip(qd, ud, vd, xd, bd)
+    assert torch.equal(IU.bitstack_forward_hip(qd, ud, vd, xd, bd), y)
+    y = y.cpu().numpy()
+    assert y.dtype == np.float16 and y.shape == (T, M)
+    assert_close(y, exact, "vs fp64")
+    if I <= 8:
+        assert_close(y, l0, "vs level-0 order")
+    w = IU.unpack_and_reconstruct_w_hip(qd, ud, vd)
+    dense = IU.linear_f16_hip(xd, w, bd).cpu().numpy()
+    assert_close(y, dense, "vs rebuilt weight x dense kernel", 2e-3, 2e-4)
+
+
+def test_walked_strips_are_declined_where_rebuild_and_dense_kernel_are_faster():
+    L = _lib.lib()
+    rebuilt = lambda M, N: M * N * 2
+    assert L.bs_workspace_bytes(8, 14336, 4096, 16, 64) == rebuilt(14336, 4096)     # 448 workgroups for 512 slots, many blocks
+    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 64) < rebuilt(14336, 4096)      # ... few blocks: taken
+    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 96) == rebuilt(14336, 4096)     # ... but not with six token tiles
+    assert L.bs_workspace_bytes(8, 4096, 14336, 16, 64) < rebuilt(4096, 14336)      # 512 workgroups
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 97) == rebuilt(4096, 4096)       # seven token tiles
+    assert L.bs_workspace_bytes(20, 4096, 4096, 16, 64) == rebuilt(4096, 4096)      # vt of 20 blocks: no room for two workgroups
+    assert L.bs_workspace_bytes(3, 4096, 4000, 16, 64) == rebuilt(4096, 4000)       # N not a multiple of 128
+
+
 @pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)
 def test_forward_few_dozen_tokens_matches_oracle(I, M, N, T, K):
     print(f"forward strips I={I} M={M} N={N} T={T} K={K}", flush=True)
