@@ -11,10 +11,14 @@
 // v_mfma_f32_16x16x16_f16 computed TRANSPOSED, D[n, m] = sum_r vt[r, n] u[m, r],
 // so that a lane ends up with four consecutive columns of one row - one nibble
 // of that row's packed sign byte - and, over a pair of patches, with a whole byte
-// (eight consecutive columns, one 16-byte store).  The sign is moved to bit 31,
-// merged into the constant 1.0f and applied with one FMA.  Signs and u of the
+// (eight consecutive columns, one 16-byte store).  A nibble addresses a 16-entry
+// table in LDS that holds its four signs as halves of +-1.0, which a mixed-precision
+// FMA (fp32 product x fp16 sign + fp32 sum) multiplies in: half a VALU instruction per
+// sign for the lookup instead of two for shifting and merging each sign bit.  Signs and u of the
 // next block are loaded while the current block is multiplied.
 #include "common.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -23,15 +27,31 @@ constexpr int VSTRIDE = 16;    // halves per column in LDS: the 16 ranks, contig
 constexpr int VGROUP_PAD = 4;  // extra halves after every 8 columns (keeps the fragment reads off each other's banks)
 constexpr int VBLOCK = RT_COLS * VSTRIDE + (RT_COLS / 8) * VGROUP_PAD;   // halves per block in LDS
 constexpr int RT_MAXB = 36;    // most blocks whose vt strip fits in LDS (36 x 4.1 KB)
+constexpr int SIGN_LUT_HALVES = 64;   // 16 nibbles x 4 signs
+#ifndef BS_REC_NSETS
+#define BS_REC_NSETS 3
+#endif
+constexpr int NSETS = BS_REC_NSETS;    // register sets of (u rows, sign words): requests run NSETS - 1 pairs ahead
 
-template <bool PACKED>
+// K16: the rank is 16 (every u fragment is one 8-byte load).  Smaller ranks pick their halves one by one behind
+// branches, and the compiler then waits for every load in flight where the branches meet: that instantiation runs
+// one pair ahead at best.
+template <bool PACKED, bool K16>
 __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
     const uint8_t *__restrict__ packed, const int8_t *__restrict__ sign,
     const half_t *__restrict__ u, const half_t *__restrict__ vt, half_t *__restrict__ w,
     int I, int M, int N, int K, int rows_per_wg) {
-    extern __shared__ __attribute__((aligned(16))) half_t vl[];   // [I][VBLOCK]: column c of a block at c * 16 + (c / 8) * 4
+    // First the 16 sign nibbles as four halves each (+1.0 for a set bit, first column in the top bit; at offset 0, so
+    // that a nibble times 8 is the address), then [I][VBLOCK]: column c of a block at c * 16 + (c / 8) * 4.
+    extern __shared__ __attribute__((aligned(128))) half_t lds_all[];
+    half_t *const lut = lds_all;
+    half_t *const vl = lds_all + SIGN_LUT_HALVES;
+    // the table's LDS address as a number: the table is 128-byte aligned, so a nibble's offset is OR-ed into it
+    typedef const __attribute__((address_space(3))) half4_t *lds_half4_ptr;
+    const uint32_t lut_base = (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) half_t *)lut);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: loop counts that depend on it stay scalar
     const int lm = lane & 15, g = lane >> 4;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  The eight
     // strips that share one 128-byte line of sign bytes must meet in ONE L2, and so
@@ -57,8 +77,9 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
     // Patches come in pairs: of a 32-column group, patch 2q takes columns 8g'..8g'+3 and patch
     // 2q+1 columns 8g'+4..8g'+7 (g' = 0..3), so that a lane (row lm, group g) ends up with EIGHT
     // consecutive columns of its row - one byte of the packed signs, one 16-byte store.
-    // Shift that brings the lane's byte of a sign word to the top (first column at bit 31):
-    const int sh_byte = 24 - 8 * g;
+    // The lane's byte of a sign word is byte g; its two nibbles, times 8, address the table:
+    // (word >> sh_hi) & 0x78 for the first four columns, (word rotated right by sh_lo) & 0x78 for the others.
+    const int sh_hi = 8 * g + 1, sh_lo = (8 * g - 3) & 31;
     // this lane's A-fragment column within a 32-column group (n-index lm of either patch, less 4 * (s & 1))
     const int acol = 8 * (lm >> 2) + (lm & 3);
     const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
@@ -74,7 +95,7 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         auto load_block = [&](int i, half4_t &b, uint4_t &sw) {
             const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
             const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
-            if (K == 16) {
+            if (K16) {
                 b = *reinterpret_cast<const half4_t *>(up);
             } else {
 #pragma unroll
@@ -87,9 +108,13 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         };
         // The (row step, block) pairs of this wave form one sequence; its loads run TWO pairs
         // ahead (one pair of work does not cover the memory latency: the waves were waiting
-        // for data two thirds of their time).
-        half4_t b_cur, b_n1, b_n2;
-        uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+        // for data two thirds of their time), into three register sets used in turn - the loop
+        // is written out three pairs at a time, so that no set is ever copied into another: a
+        // copy waits for the load it copies, which would pull every request back to one pair ahead.
+        half4_t b_set[NSETS];
+        uint4_t sw_set[NSETS];
+#pragma unroll
+        for (int k = 0; k < NSETS; k++) sw_set[k] = (uint4_t){0, 0, 0, 0};
         const int first_row = row_begin + wave * 16;
         // Requests are unconditional (behind the last pair they repeat its row step): a
         // branch around a load makes the compiler wait for every load in flight at the join.
@@ -109,8 +134,8 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                 set_row(pf_m0);
             }
         };
-        request(b_cur, sw_cur);
-        request(b_n1, sw_n1);
+#pragma unroll
+        for (int k = 0; k + 1 < NSETS; k++) request(b_set[k], sw_set[k]);
 
         // four blocks at a time, so that their loads are in flight together
         for (int q0 = 0; q0 < ib; q0 += 4) {
@@ -129,62 +154,79 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                 }
             }
         }
+        if (PACKED && tid < SIGN_LUT_HALVES) lut[tid] = ((tid >> 2) >> (3 - (tid & 3))) & 1 ? (half_t)1.f : (half_t)-1.f;
         __syncthreads();
 
-        // 16 rows per wave and step
-        for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += 64) {
+        // 16 rows per wave and step; the current pair is (rows m0.., block i)
+        // The first block of a row step starts the sums (a product, not a sum with zero): cleared accumulators
+        // would meet the running ones where the paths join, and the compiler then copies two dozen registers per block.
+        float4_t acc[8];
+        int i = 0, m0 = first_row;
+        auto consume = [&](const half4_t &b_cur, const uint4_t &swc, auto first_tag) {
+            constexpr bool FIRST = decltype(first_tag)::value;
             const int row = min(m0 + lm, M - 1);
-            float4_t acc[8];
+            const half_t *vb = vl + i * VBLOCK + aoff;
+            // all eight fragments first, and every product one patch ahead of the sign FMAs
+            // that use it: neither the LDS nor the MFMA latency sits in front of them
+            half4_t a[8];
 #pragma unroll
-            for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-            for (int i = 0; i < ib; i++) {
-                request(b_n2, sw_n2);
-                const uint4_t swc = sw_cur;      // bit 1 means +1: the product enters negated, times -1.0f
-                const half_t *vb = vl + i * VBLOCK + aoff;
-                // all eight fragments first, and every product one patch ahead of the sign FMAs
-                // that use it: neither the LDS nor the MFMA latency sits in front of them
-                half4_t a[8];
+            for (int s = 0; s < 8; s++)
+                a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
+            // the signs of a patch as four halves of +-1.0 from the table (16 entries of 8 bytes: one entry per
+            // pair of banks, equal nibbles read the same address), multiplied in by a mixed-precision FMA
+            half4_t sv[8];
+            if (PACKED) {
 #pragma unroll
-                for (int s = 0; s < 8; s++)
-                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
-                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t hi = ((swc[q] >> sh_hi) & 0x78u) | lut_base;
+                    const uint32_t lo = (__builtin_amdgcn_alignbit(swc[q], swc[q], sh_lo) & 0x78u) | lut_base;
+                    sv[2 * q] = *reinterpret_cast<lds_half4_ptr>(hi);
+                    sv[2 * q + 1] = *reinterpret_cast<lds_half4_ptr>(lo);
+                }
+            }
+            float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    const float4_t p = p_next;
-                    if (s + 1 < 8)
-                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                    if (PACKED) {
-                        uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
+            for (int s = 0; s < 8; s++) {
+                const float4_t p = p_next;
+                if (s + 1 < 8)
+                    p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                if (PACKED) {
 #pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                            acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
-                        }
-                    } else {
-                        uint32_t t = *reinterpret_cast<const uint32_t *>(
-                            sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 32 * (s >> 1) + 8 * g + 4 * (s & 1));
+                    for (int j = 0; j < 4; j++) acc[s][j] = FIRST ? p[j] * (float)sv[s][j] : __builtin_fmaf(p[j], (float)sv[s][j], acc[s][j]);
+                } else {
+                    uint32_t t = *reinterpret_cast<const uint32_t *>(
+                        sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 32 * (s >> 1) + 8 * g + 4 * (s & 1));
 #pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
-                            acc[s][j] = __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
-                        }
+                    for (int j = 0; j < 4; j++) {
+                        uint32_t sf = ((t << (24 - 8 * j)) & 0x80000000u) | 0x3F800000u;
+                        acc[s][j] = FIRST ? p[j] * __builtin_bit_cast(float, sf) : __builtin_fmaf(p[j], __builtin_bit_cast(float, sf), acc[s][j]);
                     }
                 }
-                b_cur = b_n1;
-                sw_cur = sw_n1;
-                b_n1 = b_n2;
-                sw_n1 = sw_n2;
             }
-
-            if (m0 + lm < M) {
-                half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 8 * g;
+            if (++i == ib) {
+                if (m0 + lm < M) {
+                    half_t *wp = w + (int64_t)(m0 + lm) * N + n0 + 8 * g;
 #pragma unroll
-                for (int s = 0; s < 8; s += 2) {
-                    half8_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3],
-                                 (half_t)acc[s + 1][0], (half_t)acc[s + 1][1], (half_t)acc[s + 1][2], (half_t)acc[s + 1][3]};
-                    *reinterpret_cast<half8_t *>(wp + 16 * s) = o;      // 32 columns per pair of patches
+                    for (int s = 0; s < 8; s += 2) {
+                        half8_t o = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3],
+                                     (half_t)acc[s + 1][0], (half_t)acc[s + 1][1], (half_t)acc[s + 1][2], (half_t)acc[s + 1][3]};
+                        *reinterpret_cast<half8_t *>(wp + 16 * s) = o;      // 32 columns per pair of patches
+                    }
                 }
+                i = 0;
+                m0 += 64;
+            }
+        };
+        const int n_pairs = first_row < row_end ? ((row_end - first_row + 63) / 64) * ib : 0;
+        for (int p = 0; p < n_pairs; p += NSETS) {
+#pragma unroll
+            for (int k = 0; k < NSETS; k++) {
+                if (k > 0 && p + k >= n_pairs) break;
+                request(b_set[(k + NSETS - 1) % NSETS], sw_set[(k + NSETS - 1) % NSETS]);   // the set consumed last
+                if (i == 0)
+                    consume(b_set[k], sw_set[k], std::true_type{});
+                else
+                    consume(b_set[k], sw_set[k], std::false_type{});
             }
         }
     }
@@ -232,7 +274,7 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
         // how many workgroups a CU holds), so that no second, partial wave trails behind.
         // Every workgroup re-stages its vt strip, so rows per workgroup stay a multiple of 64.
         const int strips = N / RT_COLS, strips8 = (int)bs_cdiv(strips, 8) * 8;
-        const size_t lds_need = (size_t)I * VBLOCK * sizeof(half_t);
+        const size_t lds_need = (size_t)I * VBLOCK * sizeof(half_t) + SIGN_LUT_HALVES * sizeof(half_t);   // vt images + sign table
         int per_cu = (int)((160 * 1024) / lds_need);
         if (per_cu > 8) per_cu = 8;
         if (per_cu < 1) per_cu = 1;
@@ -241,11 +283,15 @@ int launch_reconstruct(const uint8_t *packed, const int8_t *sign, const half_t *
         int rows_per_wg = (int)bs_cdiv(bs_cdiv(M, row_groups), 64) * 64;
         row_groups = (int)bs_cdiv(M, rows_per_wg);
         const size_t lds = lds_need;
-        static bs_lds_grant granted[BS_MAX_DEVICES];
-        const int st = bs_allow_lds((const void *)reconstruct_tile_kernel<PACKED>, lds, granted);
+        static bs_lds_grant granted[2][BS_MAX_DEVICES];
+        const void *kernel = K == 16 ? (const void *)reconstruct_tile_kernel<PACKED, true> : (const void *)reconstruct_tile_kernel<PACKED, false>;
+        const int st = bs_allow_lds(kernel, lds, granted[K == 16]);
         if (st != BS_OK) return st;
         dim3 grid((unsigned)bs_cdiv(strips, 8) * 8, row_groups);
-        reconstruct_tile_kernel<PACKED><<<grid, 256, lds, s>>>(packed, sign, u, vt, w, I, M, N, K, rows_per_wg);
+        if (K == 16)
+            reconstruct_tile_kernel<PACKED, true><<<grid, 256, lds, s>>>(packed, sign, u, vt, w, I, M, N, K, rows_per_wg);
+        else
+            reconstruct_tile_kernel<PACKED, false><<<grid, 256, lds, s>>>(packed, sign, u, vt, w, I, M, N, K, rows_per_wg);
     } else {
         int64_t blocks = bs_cdiv((int64_t)M * N, 256);
         if (blocks > 256 * 64) blocks = 256 * 64;

@@ -5,8 +5,9 @@
 //
 // Same decomposition as the weight rebuild (a workgroup owns a strip of 128 columns and
 // a range of rows, the strip's slice of vt of ALL blocks staged transposed in LDS, per
-// block one v_mfma_f32_16x16x16_f16 per 16 x 16 patch computed transposed, sign applied
-// as bit 31 of 1.0f in one FMA).  When the last block of a 16-row step is in, a lane
+// block one v_mfma_f32_16x16x16_f16 per 16 x 16 patch computed transposed, the signs of a
+// nibble looked up as four halves of +-1.0 and multiplied in by a mixed-precision FMA).
+// When the last block of a 16-row step is in, a lane
 // holds w[m0 + lm, 4 consecutive columns] of each patch - exactly the B operand of a
 // second v_mfma_f32_16x16x16_f16 whose A operand is x[16 tokens, the same 4 columns]
 // (read from an LDS copy of the strip's slice of x) and whose result is y[token, row]
@@ -15,7 +16,7 @@
 // [strip, T, M] (fp32); the reduce kernel of the decode path adds them in strip order
 // and applies bias and epilogue.
 //
-// Cost per 16 x 16 patch and block: the same ~14 VALU operations as the rebuild, no store
+// Cost per 16 x 16 patch and block: the same 6 to 7 VALU operations as the rebuild, no store
 // of w (two thirds of the rebuild's bytes) and no second pass that reads it back; the
 // token count only adds one MFMA per patch and 16 tokens, after the last block.
 #include "common.h"
@@ -26,6 +27,58 @@ constexpr int SF_COLS = 128;    // columns per strip
 constexpr int VSTRIDE = 16;     // halves per column of the vt image: the 16 ranks
 constexpr int VGROUP_PAD = 4;   // extra halves after every 8 columns
 constexpr int VBLOCK = SF_COLS * VSTRIDE + (SF_COLS / 8) * VGROUP_PAD;   // halves per block
+
+// The 16 sign nibbles as four halves each (+1.0 for a set bit, first column in the top bit), at the very start of
+// LDS and 128-byte aligned: a nibble times 8, OR-ed into the table's address, is where its four signs lie.  16
+// entries of 8 bytes take one pair of banks each and equal nibbles read the same address: no bank conflicts.
+constexpr int SIGN_LUT_HALVES = 64;
+typedef const __attribute__((address_space(3))) half4_t *lds_half4_ptr;
+struct SignTable {
+    uint32_t base;       // LDS address of the table
+    int sh_hi, sh_lo;    // the lane's byte of a sign word is byte g: (word >> sh_hi) & 0x78 addresses the signs of its
+                         // first four columns, (word rotated right by sh_lo) & 0x78 those of the other four
+};
+__device__ __forceinline__ SignTable make_sign_table(half_t *lut, int tid, int g) {
+    if (tid < SIGN_LUT_HALVES) lut[tid] = ((tid >> 2) >> (3 - (tid & 3))) & 1 ? (half_t)1.f : (half_t)-1.f;
+    SignTable st;
+    st.base = (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) half_t *)lut);
+    st.sh_hi = 8 * g + 1;
+    st.sh_lo = (8 * g - 3) & 31;
+    return st;
+}
+
+// Register sets of (u rows, sign words) a wave's requests rotate through: they run NSETS - 1 (row step, strip,
+// block) triples ahead.  The loops below are written out NSETS triples at a time, so that no set is ever copied
+// into another: a copy waits for the load it copies, which would pull every request back to one triple ahead.
+constexpr int NSETS = 3;
+
+// One block of a 16-row x 128-column patch row: acc[s][j] += sign * (u . vt) for the eight 16 x 16 patches.
+// vb: this lane's fragment of the block's vt image.  All eight fragments and all eight sign vectors are
+// requested first, and every product runs one patch ahead of the FMAs that use it: neither the LDS nor the
+// MFMA latency sits in front of them.
+__device__ __forceinline__ void rebuild_block(const half_t *vb, const half4_t b, const uint4_t sw, const SignTable st,
+                                              float4_t (&acc)[8]) {
+    half4_t a[8], sv[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+        a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
+    auto lookup = [&](int q) {      // the signs of patches 2q and 2q + 1
+        const uint32_t hi = ((sw[q] >> st.sh_hi) & 0x78u) | st.base;
+        const uint32_t lo = (__builtin_amdgcn_alignbit(sw[q], sw[q], st.sh_lo) & 0x78u) | st.base;
+        sv[2 * q] = *reinterpret_cast<lds_half4_ptr>(hi);
+        sv[2 * q + 1] = *reinterpret_cast<lds_half4_ptr>(lo);
+    };
+    lookup(0);
+    float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        const float4_t p = p_next;
+        if (s + 1 < 8) p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        if (s % 2 == 0 && s < 6) lookup(s / 2 + 1);   // the sign vectors of the next two patches, while these two are used
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[s][j] = __builtin_fmaf(p[j], (float)sv[s][j], acc[s][j]);
+    }
+}
 
 // TT = token tiles of 16.  A workgroup takes `sg` (1, 2, 4 or 8) neighbouring strips at once:
 // their vt slices are staged together, and per 16-row step the partial y of all of them
@@ -46,11 +99,15 @@ struct StripGroup {
     float *ssq;     // [strip groups of matrix 0][T]: sum of x^2 over the group's columns (for an RMS scale), or null
 };
 
-template <int TT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
+// K16: the rank is 16 (every u fragment is one 8-byte load).  Smaller ranks pick their halves one by one behind
+// branches, and the compiler then waits for every load in flight where the branches meet.
+template <int TT, int WAVES, bool K16>
+__global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
     const StripGroup grp, const half_t *__restrict__ x, int N, int K, int T) {
-    extern __shared__ __attribute__((aligned(16))) half_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __attribute__((aligned(128))) half_t lds_all[];
+    half_t *const lds = lds_all + SIGN_LUT_HALVES;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // the same in every lane: loop counts that depend on it stay scalar
     const int lm = lane & 15, g = lane >> 4;
     // Workgroups are dealt round-robin to the 8 XCDs.  Every matrix owns a run of block
     // indices that starts at a multiple of 8, so each XCD gets an eighth of every matrix
@@ -95,7 +152,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
 
     const int sr = tid & 15, sp = (tid >> 4) & 15;  // staging role: rank, piece of 8 columns
     const int spair = tid >> 8;                     // ... and which of the WAVES / 4 pairs staged side by side
-    const int sh_byte = 24 - 8 * g;                 // brings the lane's byte of a sign word to the top
+    const SignTable st = make_sign_table(lds_all, tid, g);
     const int acol = 8 * (lm >> 2) + (lm & 3);
     const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
 
@@ -114,7 +171,7 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
     auto load_block = [&](int i, int q, half4_t &b, uint4_t &sw) {
         const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
         const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
-        if (K == 16) {
+        if (K16) {
             b = *reinterpret_cast<const half4_t *>(up);
         } else {
 #pragma unroll
@@ -124,11 +181,15 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
         sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
     };
     // The (row step, strip, block) triples of this wave form one sequence; its sign and u loads run
-    // TWO triples ahead, and they are unconditional (behind the last triple they repeat its row
+    // NS - 1 triples ahead, and they are unconditional (behind the last triple they repeat its row
     // step): a branch around a load makes the compiler wait for every load in flight at the join,
     // which left the waves waiting for data half of their time.
-    half4_t b_cur, b_n1, b_n2;
-    uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+    // (three token tiles leave registers for two sets only)
+    constexpr int NS = TT >= 3 ? 2 : NSETS;
+    half4_t b_set[NS];
+    uint4_t sw_set[NS];
+#pragma unroll
+    for (int k = 0; k < NS; k++) sw_set[k] = (uint4_t){0, 0, 0, 0};
     int pf_i = 0, pf_q = 0, pf_m0 = first_row;      // the triple the next request is for
     set_row(pf_m0);
     auto request = [&](half4_t &b, uint4_t &sw) {
@@ -142,8 +203,8 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
             }
         }
     };
-    request(b_cur, sw_cur);
-    request(b_n1, sw_n1);
+#pragma unroll
+    for (int k = 0; k + 1 < NS; k++) request(b_set[k], sw_set[k]);
 
     // x image: token rows beyond T are zero
     for (int idx = tid; idx < TT * 16 * ns * 16; idx += NT) {
@@ -196,56 +257,31 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
     // this lane's x fragments: token lm of a tile, columns 32 (s / 2) + 8 g + 4 (s % 2) .. + 3 of patch s
     const half_t *xfrag = xl + lm * xstride + 8 * g;
 
-    for (int m0 = row_begin + wave * 16; m0 < row_end; m0 += RS) {
-        float4_t yacc[TT];
+    // the triple being consumed: rows m0.., strip q of the group, block i
+    float4_t yacc[TT], acc[8];
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-        for (int q = 0; q < ns; q++) {
-            float4_t acc[8];
+    for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
-
-            for (int i = 0; i < I; i++) {
-                request(b_n2, sw_n2);
-                const uint4_t swc = sw_cur;         // bit 1 means +1: the product enters negated, times -1.0f
-                const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
-                // all eight fragments first, and every product one patch ahead of the sign FMAs that use it
-                half4_t a[8];
+    for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    int i = 0, q = 0, m0 = first_row;
+    auto consume = [&](const half4_t &b, const uint4_t &sw) {
+        rebuild_block(vl + (q * I + i) * VBLOCK + aoff, b, sw, st, acc);
+        if (++i < I) return;
+        i = 0;
+        // y[token, row] of this strip: D[token 4g + v, row lm] = sum_k x[token, col(k)] * w[row, col(k)]
+        const half_t *xq = xfrag + q * SF_COLS;
 #pragma unroll
-                for (int s = 0; s < 8; s++)
-                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
-                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        for (int s = 0; s < 8; s++) {
+            const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
+            acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    const float4_t p = p_next;
-                    if (s + 1 < 8)
-                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                    const uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                        acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
-                    }
-                }
-                b_cur = b_n1;
-                sw_cur = sw_n1;
-                b_n1 = b_n2;
-                sw_n1 = sw_n2;
-            }
-
-            // y[token, row] of this strip: D[token 4g + v, row lm] = sum_k x[token, col(k)] * w[row, col(k)]
-            const half_t *xq = xfrag + q * SF_COLS;
-#pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-#pragma unroll
-                for (int tt = 0; tt < TT; tt++) {
-                    const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
-                    yacc[tt] = __builtin_amdgcn_mfma_f32_16x16x16f16(xf, wf, yacc[tt], 0, 0, 0);
-                }
+            for (int tt = 0; tt < TT; tt++) {
+                const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
+                yacc[tt] = __builtin_amdgcn_mfma_f32_16x16x16f16(xf, wf, yacc[tt], 0, 0, 0);
             }
         }
+        if (++q < ns) return;
+        q = 0;
         if (m0 + lm < M) {
 #pragma unroll
             for (int tt = 0; tt < TT; tt++)
@@ -254,6 +290,18 @@ __global__ __launch_bounds__(64 * WAVES, 16 / WAVES) void strip_forward_kernel(
                     const int t = 16 * tt + 4 * g + v;
                     if (t < T) part[((int64_t)group * T + t) * M + m0 + lm] = yacc[tt][v];
                 }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        m0 += RS;
+    };
+    const int n_triples = first_row < row_end ? ((row_end - first_row + RS - 1) / RS) * ns * I : 0;
+    for (int p = 0; p < n_triples; p += NS) {
+#pragma unroll
+        for (int k = 0; k < NS; k++) {
+            if (k > 0 && p + k >= n_triples) break;
+            request(b_set[(k + NS - 1) % NS], sw_set[(k + NS - 1) % NS]);   // the set consumed last
+            consume(b_set[k], sw_set[k]);
         }
     }
 }
@@ -273,11 +321,13 @@ struct WideMat {
     int I, M, sg, n_chunk, row_tiles;
 };
 
-template <int TT>
-__global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, const half_t *__restrict__ x, int N, int K, int T) {
+template <int TT, bool K16>
+__global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, const half_t *__restrict__ x, int N, int K, int T) {
     constexpr int WAVES = 8, NT = 64 * WAVES, RS = 16 * WAVES;
-    extern __shared__ __attribute__((aligned(16))) half_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __attribute__((aligned(128))) half_t lds_all[];
+    half_t *const lds = lds_all + SIGN_LUT_HALVES;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lm = lane & 15, g = lane >> 4;
     int cgroup, rt;
     {
@@ -301,7 +351,7 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
 
     const int sr = tid & 15, sp = (tid >> 4) & 15;  // staging role: rank, piece of 8 columns
     const int spair = tid >> 8;                     // ... and which of the two (strip, block) pairs staged side by side
-    const int sh_byte = 24 - 8 * g;                 // brings the lane's byte of a sign word to the top
+    const SignTable st = make_sign_table(lds_all, tid, g);
     const int acol = 8 * (lm >> 2) + (lm & 3);
     const int aoff = acol * VSTRIDE + (lm >> 2) * VGROUP_PAD + 4 * g;
 
@@ -312,7 +362,7 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
     auto load_block = [&](int i, int strip, half4_t &b, uint4_t &sw) {
         const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
         const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
-        if (K == 16) {
+        if (K16) {
             b = *reinterpret_cast<const half4_t *>(up);
         } else {
 #pragma unroll
@@ -321,10 +371,12 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
         const uint8_t *sb = packed + i * block_bytes + ((strip * SF_COLS) >> 3);
         sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
     };
-    // The (strip, block) pairs of this wave form one sequence over all its chunks; the sign and u loads run two
-    // pairs ahead, unconditionally (behind the last strip they repeat it).
-    half4_t b_cur, b_n1, b_n2;
-    uint4_t sw_cur = {0, 0, 0, 0}, sw_n1 = {0, 0, 0, 0}, sw_n2 = {0, 0, 0, 0};
+    // The (strip, block) pairs of this wave form one sequence over all its chunks; the sign and u loads run
+    // NSETS - 1 pairs ahead, unconditionally (behind the last strip they repeat it).
+    half4_t b_set[NSETS];
+    uint4_t sw_set[NSETS];
+#pragma unroll
+    for (int k = 0; k < NSETS; k++) sw_set[k] = (uint4_t){0, 0, 0, 0};
     int pf_i = 0, pf_strip = first_strip;
     auto request = [&](half4_t &b, uint4_t &sw) {
         load_block(pf_i, min(pf_strip, strips - 1), b, sw);
@@ -333,19 +385,21 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
             pf_strip++;
         }
     };
-    request(b_cur, sw_cur);
-    request(b_n1, sw_n1);
+#pragma unroll
+    for (int k = 0; k + 1 < NSETS; k++) request(b_set[k], sw_set[k]);
 
-    float4_t yacc[TT];
+    float4_t yacc[TT], acc[8];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) yacc[tt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
     const half_t *xfrag = xl + lm * xstride + 8 * g;   // token lm of a tile, columns 32 (s / 2) + 8 g + 4 (s % 2) .. + 3 of patch s
 
-    for (int ch = 0; ch < n_chunk; ch++) {
-        const int s_begin = first_strip + ch * sg;
-        const int ns = max(0, min(sg, strips - s_begin));       // the same for every thread of the workgroup
+    // x and vt images of the chunk of strips that starts at s_begin (every thread of the workgroup arrives here together)
+    auto stage = [&](int s_begin) {
+        const int ns = min(sg, strips - s_begin);
         const int n0 = s_begin * SF_COLS;
-        if (ch > 0) __syncthreads();                // everybody has finished with the previous images
+        if (s_begin != first_strip) __syncthreads();   // everybody has finished with the previous images
         // x image: token rows beyond T are zero
         for (int idx = tid; idx < TT * 16 * ns * 16; idx += NT) {
             const int t = idx / (ns * 16), piece = idx % (ns * 16);
@@ -371,48 +425,56 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
             }
         }
         __syncthreads();
+    };
 
-        for (int q = 0; q < ns; q++) {
-            float4_t acc[8];
+    // the pair being consumed: strip q of the current chunk, block i
+    int i = 0, q = 0;
+    auto consume = [&](const half4_t &b, const uint4_t &sw) {
+        rebuild_block(vl + (q * I + i) * VBLOCK + aoff, b, sw, st, acc);
+        if (++i < I) return;
+        i = 0;
+        // y[token, row] += x[token, these columns] . w[row, these columns], w rounded to fp16 as the dense path rounds it
+        const half_t *xq = xfrag + q * SF_COLS;
 #pragma unroll
-            for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
-            for (int i = 0; i < I; i++) {
-                request(b_n2, sw_n2);
-                const uint4_t swc = sw_cur;         // bit 1 means +1: the product enters negated, times -1.0f
-                const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
-                half4_t a[8];
+        for (int s = 0; s < 8; s++) {
+            const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
+            acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < 8; s++)
-                    a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
-                float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-                for (int s = 0; s < 8; s++) {
-                    const float4_t p = p_next;
-                    if (s + 1 < 8)
-                        p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                    const uint32_t t = swc[s >> 1] << (sh_byte + 4 * (s & 1));
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t sf = ((t << j) & 0x80000000u) | 0x3F800000u;
-                        acc[s][j] = __builtin_fmaf(-p[j], __builtin_bit_cast(float, sf), acc[s][j]);
-                    }
-                }
-                b_cur = b_n1;
-                sw_cur = sw_n1;
-                b_n1 = b_n2;
-                sw_n1 = sw_n2;
+            for (int tt = 0; tt < TT; tt++) {
+                const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
+                yacc[tt] = __builtin_amdgcn_mfma_f32_16x16x16f16(xf, wf, yacc[tt], 0, 0, 0);
             }
-            // y[token, row] += x[token, these columns] . w[row, these columns], w rounded to fp16 as the dense path rounds it
-            const half_t *xq = xfrag + q * SF_COLS;
+        }
+        q++;
+    };
+    for (int ch = 0; ch < n_chunk; ch++) {
+        const int s_begin = first_strip + ch * sg;
+        if (s_begin >= strips) break;                  // the same for every thread of the workgroup
+        // Staging (loads behind branches, barriers) makes the compiler wait for every load in flight, so it stays
+        // outside the loop over the pairs: once per chunk instead of once per pair.
+        stage(s_begin);
+        q = 0;
+        const int n_pairs = min(sg, strips - s_begin) * I;
+        for (int p = 0; p < n_pairs; p += NSETS) {
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-#pragma unroll
-                for (int tt = 0; tt < TT; tt++) {
-                    const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
-                    yacc[tt] = __builtin_amdgcn_mfma_f32_16x16x16f16(xf, wf, yacc[tt], 0, 0, 0);
-                }
+            for (int k = 0; k < NSETS; k++) {
+                if (k > 0 && p + k >= n_pairs) break;
+                request(b_set[(k + NSETS - 1) % NSETS], sw_set[(k + NSETS - 1) % NSETS]);   // the set consumed last
+                consume(b_set[k], sw_set[k]);
             }
+        }
+        // the next chunk starts with set 0 again: turn the sets by what this chunk's pairs left over (the copies wait
+        // for the requests in flight, as the staging of the next chunk does anyway)
+        for (int r = n_pairs % NSETS; r > 0; r--) {
+            const half4_t b0 = b_set[0];
+            const uint4_t sw0 = sw_set[0];
+#pragma unroll
+            for (int k = 0; k + 1 < NSETS; k++) {
+                b_set[k] = b_set[k + 1];
+                sw_set[k] = sw_set[k + 1];
+            }
+            b_set[NSETS - 1] = b0;
+            sw_set[NSETS - 1] = sw0;
         }
     }
     if (m0 + lm < M) {
@@ -427,6 +489,11 @@ __global__ __launch_bounds__(512, 2) void strip_wide_kernel(const WideMat mat, c
 }
 
 // Column groups and strips per chunk of the walked kernel: two workgroups per CU (LDS), about two per CU in all.
+// sign table, x image of tt token tiles, vt images of sg strips
+size_t strip_lds(int I, int tt, int sg) {
+    return (SIGN_LUT_HALVES + (size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
+}
+
 struct WidePlan {
     int tt, sg, n_chunk, col_groups, row_tiles;
     size_t lds;
@@ -443,7 +510,7 @@ WidePlan make_wide_plan(int I, int M, int N, int T) {
     const int strips = N / SF_COLS;
     p.sg = 0;
     for (int sg = 8; sg >= 1; sg >>= 1) {
-        const size_t lds = ((size_t)sg * I * VBLOCK + (size_t)p.tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
+        const size_t lds = strip_lds(I, p.tt, sg);
         if (lds * 2 <= 160 * 1024 || sg == 1) {
             p.sg = sg;
             p.lds = lds;
@@ -469,14 +536,18 @@ WidePlan make_wide_plan(int I, int M, int N, int T) {
     return p;
 }
 
-template <int TT>
-int launch_wide(const WideMat &m, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
+template <int TT, bool K16>
+int launch_wide_k(const WideMat &m, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
     static bs_lds_grant granted[BS_MAX_DEVICES];
-    const int st = bs_allow_lds((const void *)strip_wide_kernel<TT>, lds, granted);
+    const int st = bs_allow_lds((const void *)strip_wide_kernel<TT, K16>, lds, granted);
     if (st != BS_OK) return st;
-    strip_wide_kernel<TT><<<grid, 512, lds, s>>>(m, x, N, K, T);
+    strip_wide_kernel<TT, K16><<<grid, 512, lds, s>>>(m, x, N, K, T);
     BS_LAUNCH_CHECK();
     return BS_OK;
+}
+template <int TT>
+int launch_wide(const WideMat &m, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
+    return K == 16 ? launch_wide_k<TT, true>(m, grid, lds, x, N, K, T, s) : launch_wide_k<TT, false>(m, grid, lds, x, N, K, T, s);
 }
 
 struct StripPlan {
@@ -486,9 +557,6 @@ struct StripPlan {
 
 int token_tiles(int T) { return (T + 15) / 16; }
 
-size_t strip_lds(int I, int tt, int sg) {
-    return ((size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
-}
 
 // Workgroups of 8 waves (two per CU): they share one vt image, so a CU holds 16 waves with half the
 // LDS four-wave workgroups would need (at 16 blocks two of those, 8 waves, were all a CU could hold).
@@ -531,19 +599,20 @@ StripPlan make_strip_plan(int I, int M, int N, int T) {
     return best;
 }
 
-template <int TT, int WAVES>
+template <int TT, int WAVES, bool K16>
 int launch_ttw(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
     static bs_lds_grant granted[BS_MAX_DEVICES];
-    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT, WAVES>, lds, granted);
+    const int st = bs_allow_lds((const void *)strip_forward_kernel<TT, WAVES, K16>, lds, granted);
     if (st != BS_OK) return st;
-    strip_forward_kernel<TT, WAVES><<<grid, 64 * WAVES, lds, s>>>(grp, x, N, K, T);
+    strip_forward_kernel<TT, WAVES, K16><<<grid, 64 * WAVES, lds, s>>>(grp, x, N, K, T);
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
 
 template <int TT>
 int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int N, int K, int T, hipStream_t s) {
-    return launch_ttw<TT, STRIP_WAVES>(grp, grid, lds, x, N, K, T, s);
+    return K == 16 ? launch_ttw<TT, STRIP_WAVES, true>(grp, grid, lds, x, N, K, T, s)
+                   : launch_ttw<TT, STRIP_WAVES, false>(grp, grid, lds, x, N, K, T, s);
 }
 
 }  // namespace
