@@ -339,24 +339,33 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // D[r, m]: the lane holds ranks 4g..4g+3 of row (tile jr, lm).  Subtract the correction
     // (summed over waves in a fixed order), scale by u, add the four lane groups, write the
     // partial row sum, start the next row from zero.
+    // The u rows a flush multiplies by are requested one unit earlier (before the last unit of the row is
+    // multiplied): requested inside the flush, every wave sat out their whole latency there.
+    half4_t uc[R];
+    auto request_u = [&](int rowid) {
+        const int i = rowid / row_tiles, rt = rowid % row_tiles;
+#pragma unroll
+        for (int jr = 0; jr < R; jr++) {
+            const int row = min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
+            const half_t *up = u + ((int64_t)i * M + row) * K;
+            if (K == 16) {
+                uc[jr] = *reinterpret_cast<const half4_t *>(up + 4 * g);
+            } else {
+                // (ranks beyond K repeat rank K - 1 and are zeroed: no branch around a load)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const half_t val = up[min(4 * g + v, K - 1)];
+                    uc[jr][v] = (4 * g + v < K) ? val : (half_t)0;
+                }
+            }
+        }
+    };
     int flush_parity = 0;
     auto flush = [&](int rowid, bool row_done) {
         // two flushes can follow each other with no barrier in between, so the exchange area alternates
         float *cx = corrl + flush_parity * (MX_WAVES * 16);
         flush_parity ^= 1;
         const int i = rowid / row_tiles, rt = rowid % row_tiles;
-        half4_t uc[R];
-#pragma unroll
-        for (int jr = 0; jr < R; jr++) {
-            const int row = min(rt * RW + (wave * R + jr) * 16 + lm, M - 1);
-            const half_t *up = u + ((int64_t)i * M + row) * K + 4 * g;
-            if (K == 16) {
-                uc[jr] = *reinterpret_cast<const half4_t *>(up);
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; v++) uc[jr][v] = (4 * g + v < K) ? up[v] : (half_t)0;
-            }
-        }
         if (lm == 0) *reinterpret_cast<float4_t *>(cx + wave * 16 + 4 * g) = corr;
         __syncthreads();
         const int slot = wg - sp.owner(rowid * n_units);
@@ -397,33 +406,19 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
 #pragma unroll
         for (int jr = 0; jr < R; jr++) w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
     }
-    uint32_t warm0;      // loaded for its side effect only (the line ends up in L2)
-    {
-        const int lrow = (u_end - 1) / n_units, fi = lrow / row_tiles, frt = lrow % row_tiles;
-        const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
-        warm0 = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
-    }
     produce_write(0);
     __syncthreads();
-    asm volatile("" ::"v"(warm0));
 
     // ---- steady state ----------------------------------------------------------------------------
     int buf = 0;
-    uint32_t warm_in = 0;
     for (int unit = u_begin; unit + 1 < u_end; unit++) {
         const bool crossing = c + 1 == n_units;     // the next unit starts another row of units
         const int cn = crossing ? 0 : c + 1;
-        if (crossing) {
-            // the row ends with this unit: pull its u rows towards L2 now (one dword per row, value unused)
-            const int fi = rowid / row_tiles, frt = rowid % row_tiles;
-            const int frow = min(frt * RW + wave * (R * 16) + (lane & (R * 16 - 1)), M - 1);
-            warm_in = *reinterpret_cast<const uint32_t *>(u + ((int64_t)fi * M + frow) * K);
-        }
+        if (crossing) request_u(rowid);             // the row ends with this unit
         set_unit(rowid + (crossing ? 1 : 0), cn, crossing);
         produce_issue(cn);
         __builtin_amdgcn_sched_barrier(0);
         consume(buf);
-        asm volatile("" ::"v"(warm_in));
         produce_write(buf ^ 1);
         __syncthreads();
         if (crossing) {
@@ -434,6 +429,8 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         buf ^= 1;
     }
     // ---- drain ---------------------------------------------------------------------------------------
+    request_u(rowid);
+    __builtin_amdgcn_sched_barrier(0);
     consume(buf);          // (its refill requests repeat the last unit's addresses: valid, unused)
     flush(rowid, u_end % n_units == 0);
 }
