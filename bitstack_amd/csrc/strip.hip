@@ -27,6 +27,10 @@ constexpr int SF_COLS = 128;    // columns per strip
 constexpr int VSTRIDE = 16;     // halves per column of the vt image: the 16 ranks
 constexpr int VGROUP_PAD = 4;   // extra halves after every 8 columns
 constexpr int VBLOCK = SF_COLS * VSTRIDE + (SF_COLS / 8) * VGROUP_PAD;   // halves per block
+// Extra halves per token row of the x image: rows then start two banks apart, so the 16 tokens a quarter wave reads
+// (8 bytes each, the same columns) fall on 32 different banks.  (With 8, tokens t and t + 8 shared their banks.)
+// Rows are 8-byte aligned only: the image is written and read in pieces of four halves.
+constexpr int XPAD = 4;
 
 // The 16 sign nibbles as four halves each (+1.0 for a set bit, first column in the top bit), at the very start of
 // LDS and 128-byte aligned: a nibble times 8, OR-ed into the table's address, is where its four signs lie.  16
@@ -132,7 +136,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
     const half_t *__restrict__ vt = mat.vt;
     float *__restrict__ part = mat.part;
     const int I = mat.I, M = mat.M, sg = mat.sg, rows_per_wg = mat.rows_per_wg;
-    const int xstride = sg * SF_COLS + 8;           // halves per token row of the x image
+    const int xstride = sg * SF_COLS + XPAD;        // halves per token row of the x image
     half_t *xl = lds;                               // [TT * 16][xstride]
     half_t *vl = lds + TT * 16 * xstride;           // [sg][I][VBLOCK]
     int group, row_begin;
@@ -211,7 +215,8 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
         const int t = idx / (ns * 16), piece = idx % (ns * 16);
         half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (t < T) v = *reinterpret_cast<const half8_t *>(x + (int64_t)t * N + n0 + 8 * piece);
-        *reinterpret_cast<half8_t *>(xl + t * xstride + 8 * piece) = v;
+        *reinterpret_cast<half4_t *>(xl + t * xstride + 8 * piece) = (half4_t){v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<half4_t *>(xl + t * xstride + 8 * piece + 4) = (half4_t){v[4], v[5], v[6], v[7]};
     }
     // vt slices, four (strip, block) pairs at a time so that their loads are in flight together
     constexpr int SIDE = WAVES / 4;                 // 256 threads stage one (strip, block) pair
@@ -242,9 +247,12 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
             float q = 0.f;
             if (t < TT * 16) {
                 for (int c = sub * 8; c < ns * SF_COLS; c += 64) {
-                    const half8_t v = *reinterpret_cast<const half8_t *>(xl + t * xstride + c);
+                    const half4_t v0 = *reinterpret_cast<const half4_t *>(xl + t * xstride + c);
+                    const half4_t v1 = *reinterpret_cast<const half4_t *>(xl + t * xstride + c + 4);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+                    for (int e = 0; e < 4; e++) q += (float)v0[e] * (float)v0[e];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) q += (float)v1[e] * (float)v1[e];
                 }
             }
             q += __shfl_xor(q, 1, 64);
@@ -341,7 +349,7 @@ __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, c
     const half_t *__restrict__ u = mat.u;
     const half_t *__restrict__ vt = mat.vt;
     const int I = mat.I, M = mat.M, sg = mat.sg, n_chunk = mat.n_chunk;
-    const int xstride = sg * SF_COLS + 8;           // halves per token row of the x image
+    const int xstride = sg * SF_COLS + XPAD;        // halves per token row of the x image
     half_t *xl = lds;                               // [TT * 16][xstride]
     half_t *vl = lds + TT * 16 * xstride;           // [sg][I][VBLOCK]
     const int strips = N / SF_COLS;
@@ -405,7 +413,8 @@ __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, c
             const int t = idx / (ns * 16), piece = idx % (ns * 16);
             half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
             if (t < T) v = *reinterpret_cast<const half8_t *>(x + (int64_t)t * N + n0 + 8 * piece);
-            *reinterpret_cast<half8_t *>(xl + t * xstride + 8 * piece) = v;
+            *reinterpret_cast<half4_t *>(xl + t * xstride + 8 * piece) = (half4_t){v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<half4_t *>(xl + t * xstride + 8 * piece + 4) = (half4_t){v[4], v[5], v[6], v[7]};
         }
         // vt slices, four (strip, block) pairs per thread at a time so that their loads are in flight together
         for (int q0 = 0; q0 < ns * I; q0 += 8) {
@@ -491,7 +500,7 @@ __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, c
 // Column groups and strips per chunk of the walked kernel: two workgroups per CU (LDS), about two per CU in all.
 // sign table, x image of tt token tiles, vt images of sg strips
 size_t strip_lds(int I, int tt, int sg) {
-    return (SIGN_LUT_HALVES + (size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + 8)) * sizeof(half_t);
+    return (SIGN_LUT_HALVES + (size_t)sg * I * VBLOCK + (size_t)tt * 16 * (sg * SF_COLS + XPAD)) * sizeof(half_t);
 }
 
 struct WidePlan {
