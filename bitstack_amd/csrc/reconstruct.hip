@@ -28,10 +28,7 @@ constexpr int VGROUP_PAD = 4;  // extra halves after every 8 columns (keeps the 
 constexpr int VBLOCK = RT_COLS * VSTRIDE + (RT_COLS / 8) * VGROUP_PAD;   // halves per block in LDS
 constexpr int RT_MAXB = 36;    // most blocks whose vt strip fits in LDS (36 x 4.1 KB)
 constexpr int SIGN_LUT_HALVES = 64;   // 16 nibbles x 4 signs
-#ifndef BS_REC_NSETS
-#define BS_REC_NSETS 3
-#endif
-constexpr int NSETS = BS_REC_NSETS;    // register sets of (u rows, sign words): requests run NSETS - 1 pairs ahead
+constexpr int NSETS = 3;       // register sets of (u rows, sign words): requests run NSETS - 1 pairs ahead (four to six sets: no faster)
 
 // K16: the rank is 16 (every u fragment is one 8-byte load).  Smaller ranks pick their halves one by one behind
 // branches, and the compiler then waits for every load in flight where the branches meet: that instantiation runs
