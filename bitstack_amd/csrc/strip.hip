@@ -508,7 +508,7 @@ struct WidePlan {
     size_t lds;
     bool worth;      // expected to beat rebuild + dense kernel
 };
-// Up to six token tiles two workgroups share a CU (118-125 registers); seven and eight tiles take 133 and 159, one
+// Up to six token tiles two workgroups share a CU (122-128 registers); seven and eight tiles would need 133 and 159, one
 // workgroup per CU, and lose to rebuild + dense kernel on every large shape.
 constexpr int WIDE_MIN_T = 49, WIDE_MAX_T = 96;
 
