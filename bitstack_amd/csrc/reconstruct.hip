@@ -28,7 +28,6 @@ constexpr int VGROUP_PAD = 4;  // extra halves after every 8 columns (keeps the 
 constexpr int VBLOCK = RT_COLS * VSTRIDE + (RT_COLS / 8) * VGROUP_PAD;   // halves per block in LDS
 constexpr int RT_MAXB = 36;    // most blocks whose vt strip fits in LDS (36 x 4.1 KB)
 constexpr int SIGN_LUT_HALVES = 64;   // 16 nibbles x 4 signs
-constexpr int NSETS = 3;       // register sets of (u rows, sign words): requests run NSETS - 1 pairs ahead (four to six sets: no faster)
 
 // K16: the rank is 16 (every u fragment is one 8-byte load).  Smaller ranks pick their halves one by one behind
 // branches, and the compiler then waits for every load in flight where the branches meet: that instantiation runs
@@ -88,8 +87,8 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
         // the very first block before the vt strip is staged
         // Addresses are a wave-uniform 64-bit base (the block: scalar arithmetic) plus a 32-bit
         // offset per lane that depends on the row only and is renewed once per row step.
-        uint32_t off_u, off_s;                      // bytes: this lane's u row (its four ranks) and sign row
-        auto load_block = [&](int i, half4_t &b, uint4_t &sw) {
+        uint32_t off_u;                             // bytes: this lane's u row (its four ranks)
+        auto load_u = [&](int i, half4_t &b) {
             const char *ub = reinterpret_cast<const char *>(u) + (int64_t)i * M * K * 2;
             const half_t *up = reinterpret_cast<const half_t *>(ub + off_u);
             if (K16) {
@@ -98,41 +97,65 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
 #pragma unroll
                 for (int j = 0; j < 4; j++) b[j] = (4 * g + j < K) ? up[j] : (half_t)0;
             }
-            if (PACKED) {
-                const uint8_t *sb = packed + i * block_bytes + (n0 >> 3);
-                sw = *reinterpret_cast<const uint4_t *>(sb + off_s);
-            }
         };
-        // The (row step, block) pairs of this wave form one sequence; its loads run TWO pairs
-        // ahead (one pair of work does not cover the memory latency: the waves were waiting
-        // for data two thirds of their time), into three register sets used in turn - the loop
-        // is written out three pairs at a time, so that no set is ever copied into another: a
-        // copy waits for the load it copies, which would pull every request back to one pair ahead.
-        half4_t b_set[NSETS];
-        uint4_t sw_set[NSETS];
-#pragma unroll
-        for (int k = 0; k < NSETS; k++) sw_set[k] = (uint4_t){0, 0, 0, 0};
+        // The (row step, block) pairs of this wave form one sequence.  u rows are requested pair by pair, three pairs
+        // ahead, into four register sets used in turn (the loop is written out eight pairs at a time, so that no set is
+        // ever copied into another: a copy waits for the load it copies).  Sign words are requested FOUR PAIRS PER
+        // INSTRUCTION: lane group g loads the 16 bytes of pair 4 q + g of the sequence (its row's sign bytes of this
+        // strip in that pair's block), and the pair that is being multiplied fetches its words from the group that
+        // holds them with four cross-lane reads.  Loaded pair by pair, all four lane groups requested the same 16
+        // bytes per row, and a load instruction costs the memory pipeline its 16 rows' lines whatever it brings.
+        half4_t b_set[4];
+        uint4_t quad[2];
         const int first_row = row_begin + wave * 16;
         // Requests are unconditional (behind the last pair they repeat its row step): a
         // branch around a load makes the compiler wait for every load in flight at the join.
         const int last_m0 = first_row + ((max(row_end - first_row, 1) - 1) / 64) * 64;
-        int pf_i = 0, pf_m0 = first_row;           // the pair the next request is for
+        int pf_i = 0, pf_m0 = first_row;           // the pair the next u request is for
         auto set_row = [&](int m0) {
             const int row = min(min(m0, last_m0) + lm, M - 1);
             off_u = (uint32_t)(row * K + 4 * g) * 2u;
-            off_s = (uint32_t)row * (uint32_t)row_bytes;
         };
         set_row(pf_m0);
-        auto request = [&](half4_t &b, uint4_t &sw) {
-            load_block(i0 + pf_i, b, sw);
+        auto request_u = [&](half4_t &b) {
+            load_u(i0 + pf_i, b);
             if (++pf_i == ib) {
                 pf_i = 0;
                 pf_m0 += 64;
                 set_row(pf_m0);
             }
         };
+        // the pair this lane loads for the next quad: block ql_i of the row step at ql_m0 (per lane: the groups differ)
+        int ql_i = g, ql_m0 = first_row;
+        auto wrap_quad = [&]() {
 #pragma unroll
-        for (int k = 0; k + 1 < NSETS; k++) request(b_set[k], sw_set[k]);
+            for (int r = 0; r < 4; r++)
+                if (ql_i >= ib) {
+                    ql_i -= ib;
+                    ql_m0 += 64;
+                }
+        };
+        wrap_quad();
+        auto request_quad = [&](uint4_t &qd) {
+            if (PACKED) {
+                const int row = min(min(ql_m0, last_m0) + lm, M - 1);
+                qd = *reinterpret_cast<const uint4_t *>(packed + (int64_t)(i0 + ql_i) * block_bytes + (n0 >> 3) + (int64_t)row * row_bytes);
+            }
+            ql_i += 4;
+            wrap_quad();
+        };
+        // the sign words of pair `sel` (0..3) of a quad, for every lane group
+        auto sign_words = [&](const uint4_t &qd, int sel) {
+            const int from = (16 * sel + lm) * 4;
+            uint4_t r;
+#pragma unroll
+            for (int d = 0; d < 4; d++) r[d] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)qd[d]);
+            return r;
+        };
+        quad[0] = quad[1] = (uint4_t){0, 0, 0, 0};
+        request_quad(quad[0]);
+#pragma unroll
+        for (int k = 0; k < 3; k++) request_u(b_set[k]);
 
         // four blocks at a time, so that their loads are in flight together
         for (int q0 = 0; q0 < ib; q0 += 4) {
@@ -215,15 +238,18 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
             }
         };
         const int n_pairs = first_row < row_end ? ((row_end - first_row + 63) / 64) * ib : 0;
-        for (int p = 0; p < n_pairs; p += NSETS) {
+        for (int p = 0; p < n_pairs; p += 8) {
 #pragma unroll
-            for (int k = 0; k < NSETS; k++) {
-                if (k > 0 && p + k >= n_pairs) break;
-                request(b_set[(k + NSETS - 1) % NSETS], sw_set[(k + NSETS - 1) % NSETS]);   // the set consumed last
+            for (int idx = 0; idx < 8; idx++) {
+                if (idx > 0 && p + idx >= n_pairs) break;
+                const int h = idx >> 2, k = idx & 3;
+                if (k == 0) request_quad(quad[h ^ 1]);          // the next quad, into the set consumed last
+                request_u(b_set[(k + 3) & 3]);
+                const uint4_t swc = sign_words(quad[h], k);
                 if (i == 0)
-                    consume(b_set[k], sw_set[k], std::true_type{});
+                    consume(b_set[k], swc, std::true_type{});
                 else
-                    consume(b_set[k], sw_set[k], std::false_type{});
+                    consume(b_set[k], swc, std::false_type{});
             }
         }
     }
