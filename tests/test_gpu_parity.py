@@ -87,7 +87,11 @@ def test_pack_bit_exact_and_round_trip(shape):
 # --------------------------------------------------------------- reconstruct
 RECON_CASES = [(1, 64, 128, 16), (3, 64, 256, 16), (2, 50, 128, 16), (4, 256, 512, 16),
                (2, 64, 128, 7), (1, 64, 128, 1), (2, 40, 72, 16), (3, 33, 100, 5),
-               (8, 1024, 4096, 16)]
+               (8, 1024, 4096, 16),
+               # block counts that are not multiples of the four pairs a sign load brings, many row steps per wave,
+               # ragged row counts, the most blocks the tiled kernel takes
+               (5, 700, 256, 16), (7, 1000, 384, 16), (1, 2048, 1024, 16), (36, 200, 128, 16), (6, 4096, 4096, 16),
+               (3, 130, 128, 3), (9, 14336, 128, 16)]
 
 
 @pytest.mark.parametrize("I,M,N,K", RECON_CASES)
