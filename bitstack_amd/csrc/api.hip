@@ -32,10 +32,14 @@ static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 // Which kernel multiplies the rebuilt weight: 0 by token count, 1 always linear_f16_kernel, 2 hipBLASLt
 // wherever it takes the shape (bs_set_dense_kernel, for tests and benchmarks).
 static int g_dense_kernel = 0;
-// From this many tokens on the library's kernels are the faster ones on the layer shapes measured (1024 x 4096 ..
-// 14336 x 4096 with 8 blocks, rebuild included, the four layers run in turn): 384 -> 399 useful TFLOP/s at 512
-// tokens, 662 -> 840 at 2048; at 128 and 256 tokens neither is ahead on every shape.
-constexpr int DENSE_LIBRARY_MIN_T = 512;
+// From this many tokens on the library's kernels are the faster ones behind the rebuild on the layer shapes measured
+// (1024 x 4096 .. 14336 x 4096 with 8 blocks, rebuild included, the four layers run in turn so that no layer finds its
+// operands in cache; microseconds over the four, linear_f16_kernel / library): 64 tokens 256-268 / 243-247 (only
+// 14336 x 4096 rebuilds there), 128 tokens 326-336 / 304-307, 256 tokens 325-344 / 312-314, 448 tokens 397-409 /
+// 373-374, 2048 tokens 662 / 840 useful TFLOP/s.  The library's choice of kernel is poor at a few token counts (160 and
+// 192 tokens on 4096 x 14336: 144-154 against 130-139), where the sums come out level.  Below, no shape measured
+// rebuilds a weight that the strip kernels would not take, and linear_f16_kernel's small tiles serve.
+constexpr int DENSE_LIBRARY_MIN_T = 49;
 
 static bool dense_wants_library(int M, int N, int T) {
     if (g_dense_kernel == BS_DENSE_OWN || M % 8 != 0 || N % 8 != 0) return false;

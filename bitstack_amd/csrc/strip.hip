@@ -506,7 +506,7 @@ size_t strip_lds(int I, int tt, int sg) {
 struct WidePlan {
     int tt, sg, n_chunk, col_groups, row_tiles;
     size_t lds;
-    bool worth;      // expected to beat rebuild + dense kernel
+    bool worth;      // expected to beat rebuild + dense product
 };
 // Up to six token tiles two workgroups share a CU (122-128 registers); seven and eight tiles would need 133 and 159, one
 // workgroup per CU, and lose to rebuild + dense kernel on every large shape.
@@ -534,14 +534,17 @@ WidePlan make_wide_plan(int I, int M, int N, int T) {
     if (cg < 1) cg = 1;
     p.n_chunk = (int)bs_cdiv(chunks, cg);
     p.col_groups = (int)bs_cdiv(chunks, p.n_chunk);
-    // Measured against rebuild + dense kernel (8B layer shapes, layers alternating): per block both cost about the
-    // same, but the walked kernel saves the round trip of the weight through memory (37 against 49-78 us of fixed
-    // cost on the large shapes), so it wins - by 1.2-1.7x - wherever its workgroups fill the chip, and with few
-    // blocks and up to 80 tokens also where they do not (14336 rows: 448 workgroups for 512 slots).
+    // Measured against rebuild + vendor GEMM (8B layer shapes, layers alternating): per block both cost about the
+    // same, but the walked kernel saves the round trip of the weight through memory, so it wins - by up to 1.3x -
+    // wherever its workgroups fill the chip (1024 x 4096 with 8 blocks at 64 tokens 20 against 25 us, 4096 x 14336
+    // 93 against 106) and loses where they do not (14336 x 4096, 448 workgroups for 512 slots: 90 against 74 us with
+    // 6 blocks at 64 tokens, level with 3).  The exception is a matrix wider than tall with few blocks: the GEMM behind
+    // its rebuild has few output tiles and a long inner dimension, and the walked kernel stays ahead at 448 workgroups
+    // too (4096 x 14336 at 49 tokens: 50 against 60-66 us with 3 blocks, 71 against 78-84 with 6).
     const int grid = p.row_tiles * p.col_groups;
     // (up to one workgroup per CU nothing is uneven; beyond, the busiest CU holds a whole number of rounds of two)
     const double fill = grid <= slots / 2 ? 1.0 : (double)grid / (double)(bs_cdiv(grid, slots) * slots);
-    p.worth = fill >= 0.95 || (I <= 6 && p.tt <= 5);
+    p.worth = fill >= 0.95 || (M < N && I <= 6 && p.tt <= 5);
     return p;
 }
 

@@ -125,10 +125,10 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * (more than 96 tokens, or N not a multiple of 128) need more and are refused.
  * All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (different streams, different host threads) race; calls on one
- * stream are ordered and safe.  Same results as bs_forward, bit for bit; from
- * 512 tokens on as bs_forward under bs_set_dense_kernel(BS_DENSE_OWN), because
- * the dense product here always runs this library's own kernel (the vendor
- * GEMM needs scratch of its own and allocates when it is set up).
+ * stream are ordered and safe.  Same results as bs_forward, bit for bit; where
+ * a weight is rebuilt, as bs_forward under bs_set_dense_kernel(BS_DENSE_OWN),
+ * because the dense product here always runs this library's own kernel (the
+ * vendor GEMM needs scratch of its own and allocates when it is set up).
  */
 #define BS_STATIC_SCRATCH_BYTES (64 << 20)
 int bs_forward_static(const uint8_t *packed, const void *u, const void *vt, const void *x,
@@ -171,7 +171,7 @@ int bs_set_decode_kernel(int mode);
 /*
  * Test and benchmark hook: which kernel multiplies the rebuilt weight in
  * bs_forward's large-T path.  0 = by token count (the default: this library's
- * linear_f16 kernels below 512 tokens, hipBLASLt from there on),
+ * linear_f16 kernels below 49 tokens, hipBLASLt from there on),
  * BS_DENSE_OWN = always this library's kernels, BS_DENSE_LIBRARY = hipBLASLt
  * wherever it takes the shape (M and N multiples of 8).  hipBLASLt is opened
  * at run time; where it is missing or has no kernel for a shape the call runs

@@ -287,7 +287,7 @@ STRIP_CASES = [(1, 16, 128, 5, 16), (3, 100, 384, 9, 16), (2, 65, 1152, 17, 7), 
 # token tiles, ranks below 16, one strip and several per chunk (few blocks leave room in LDS), several chunks per
 # workgroup, row counts whose workgroups do not fill the chip (few blocks: still taken), one column group and many
 WIDE_CASES = [(2, 128, 128, 49, 16), (3, 1000, 1152, 64, 16), (1, 4096, 4096, 96, 16), (8, 4096, 4096, 65, 16),
-              (3, 14336, 4096, 80, 16), (2, 4096, 14336, 50, 16), (5, 333, 640, 77, 5), (12, 1024, 4096, 96, 16),
+              (3, 8192, 4096, 80, 16), (2, 4096, 14336, 50, 16), (5, 333, 640, 77, 5), (12, 1024, 4096, 96, 16),
               (4, 130, 2432, 81, 12), (6, 2000, 1024, 49, 1)]
 
 
@@ -318,14 +318,14 @@ def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K):
 
 def test_walked_strips_are_declined_where_rebuild_and_dense_kernel_are_faster():
     L = _lib.lib()
-    rebuilt = lambda M, N: M * N * 2
-    assert L.bs_workspace_bytes(8, 14336, 4096, 16, 64) == rebuilt(14336, 4096)     # 448 workgroups for 512 slots, many blocks
-    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 64) < rebuilt(14336, 4096)      # ... few blocks: taken
-    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 96) == rebuilt(14336, 4096)     # ... but not with six token tiles
+    rebuilt = lambda M, N: M * N * 2                    # (+ the vendor GEMM's scratch where that multiplies it)
+    assert L.bs_workspace_bytes(8, 14336, 4096, 16, 64) >= rebuilt(14336, 4096)     # 448 workgroups for 512 slots
+    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 64) >= rebuilt(14336, 4096)     # ... and few blocks
+    assert L.bs_workspace_bytes(3, 8192, 4096, 16, 64) < rebuilt(8192, 4096)        # 512 workgroups: taken
     assert L.bs_workspace_bytes(8, 4096, 14336, 16, 64) < rebuilt(4096, 14336)      # 512 workgroups
-    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 97) == rebuilt(4096, 4096)       # seven token tiles
-    assert L.bs_workspace_bytes(20, 4096, 4096, 16, 64) == rebuilt(4096, 4096)      # vt of 20 blocks: no room for two workgroups
-    assert L.bs_workspace_bytes(3, 4096, 4000, 16, 64) == rebuilt(4096, 4000)       # N not a multiple of 128
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 97) >= rebuilt(4096, 4096)       # seven token tiles
+    assert L.bs_workspace_bytes(20, 4096, 4096, 16, 64) >= rebuilt(4096, 4096)      # vt of 20 blocks: no room for two workgroups
+    assert L.bs_workspace_bytes(3, 4096, 4000, 16, 64) >= rebuilt(4096, 4000)       # N not a multiple of 128
 
 
 @pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)
@@ -714,7 +714,7 @@ def _random_forced_cases(n, seed):
         elif kind == 3:    # rebuild + dense, ragged everything
             N = 8 * int(rng.integers(1, 300)); M = int(rng.integers(1, 1500)); T = int(rng.integers(1, 700)); I = int(rng.integers(1, 6))
         else:              # either side of the token count where the vendor GEMM takes over
-            N = 1024 * int(rng.integers(1, 5)); M = 512 * int(rng.integers(1, 9)); T = int(rng.choice([1, 2, 511, 512, 600, 1024])); I = int(rng.integers(1, 10))
+            N = 1024 * int(rng.integers(1, 5)); M = 512 * int(rng.integers(1, 9)); T = int(rng.choice([1, 2, 48, 49, 600, 1024])); I = int(rng.integers(1, 10))
         cases.append((I, M, N, T, int(rng.choice([16, 16, 16, 12, 5, 1])), int(rng.integers(0, 3)), int(rng.integers(0, 3))))
     return cases
 
