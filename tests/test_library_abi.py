@@ -76,8 +76,9 @@ def test_workspace_bytes(L):
     assert L.bs_workspace_bytes(8, 4096, 4096, 16, 0) == 0
     assert L.bs_workspace_bytes(8, 4096, 4100, 16, 1) == -2
     assert L.bs_workspace_bytes(8, 4096, 4096, 20, 1) == -3
-    # prefill and odd shapes rebuild the fp16 weight
-    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2
+    # prefill and odd shapes rebuild the fp16 weight (from 49 tokens followed by 64 MiB for the vendor GEMM)
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2 + (64 << 20)
+    assert L.bs_workspace_bytes(8, 4096, 4104, 16, 20) == 4096 * 4104 * 2
     assert L.bs_workspace_bytes(2, 64, 72, 16, 1) == ((64 * 72 * 2 + 255) // 256) * 256
     # decode keeps fp32 partial row sums: a multiple of T * M * 4, far below the weight
     for T in (1, 4):
