@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256, 4) void reconstruct_tile_kernel(
                     p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b_cur, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 if (PACKED) {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) acc[s][j] = FIRST ? p[j] * (float)sv[s][j] : __builtin_fmaf(p[j], (float)sv[s][j], acc[s][j]);
+                    for (int j = 0; j < 4; j++) acc[s][j] = __builtin_fmaf(p[j], (float)sv[s][j], FIRST ? 0.f : acc[s][j]);   // (a plain product would not become a mixed-precision instruction)
                 } else {
                     uint32_t t = *reinterpret_cast<const uint32_t *>(
                         sign + ((int64_t)(i0 + i) * M + row) * N + n0 + 32 * (s >> 1) + 8 * g + 4 * (s & 1));
