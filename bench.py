@@ -563,7 +563,7 @@ def main():
         b16 = sum(L.bytes for L in l16)
         t16 = sum(per16) * 1e-3
         out["t16"] = {"GBps": round(b16 / t16 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b16 / t16 / 1e9 / HBM_PEAK_GBS, 2),
-                      "kernel": "strip_forward_kernel<1,8> + gemv_reduce_kernel"}
+                      "kernel": "strip_forward_kernel<1,8> + gemv_reduce_flat_kernel"}
         detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 16, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l16, per16)]
         del l16

@@ -407,24 +407,19 @@ __global__ __launch_bounds__(64 * WAVES, (T == 1 ? (WAVES == 16 ? 1 : WAVES == 4
     flush(rowid, u_end % nch == 0);
 }
 
-// y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ) where k
-// runs over the workgroups whose unit range touched (block i, row tile of m), in
-// ascending order.  32 outputs of one row tile per workgroup; eight threads per
-// output take every eighth block (their loads are independent) and are combined
-// through LDS in a fixed order.
+// y[t, off + m] = epilogue( fp16( sum_i sum_k part[i, k, t, m] + bias[m] ) ): every one of the I * kmax
+// slots of an output holds a number (the decode kernels zero-fill the slots nobody needed; the strip
+// kernels write one partial per strip group, I = groups and kmax = 1), added up in a fixed order.
 // Epilogues (applied to the fp16-rounded sums, the way separate fp16 ops would):
 //   EPI_NONE      the matrices' outputs side by side in one row of `ldy` halves
 //   EPI_RESIDUAL  the same plus residual[t, off + m]
 //   EPI_SWIGLU    two matrices of equal M: silu(first) * second, one row of M
-constexpr int RED_OUT = 32, RED_SL = 8, RED_MAXBLOCKS = 1024;
-constexpr int RED_BATCH = 4;      // partial loads in flight per thread (eight were slower: the loads of dead slots are issued all the same)   // the last one is a sanity limit on the block count
+constexpr int RED_MAXBLOCKS = 1024;      // a sanity limit on the block count
 
 struct RedMat {
     const float *part;
     const half_t *bias;
-    int I, M, row_tiles, kmax, y_off, first_block;
-    Split sp;
-    int pair;       // as GemvMat::pair: two workgroups per place in the partition, slots 2k and 2k + 1
+    int I, M, kmax, y_off, first_block;
 };
 struct RedGroup {
     RedMat m[GEMV_MAX_GROUP];
@@ -441,153 +436,10 @@ struct RedGroup {
     int ssq_n;
 };
 
-// Sum of the partials of output m of one matrix that this thread's slice covers.
-// The (block, slot) pairs are numbered i * kmax + k and slice ks takes every
-// RED_SL-th of them, RED_BATCH at a time: slots that are not live (k beyond the number of
-// workgroups that touched this row tile of block i, `nks[i]`, worked out once per
-// workgroup) are loaded all the same (the slots exist in the workspace) and masked, so
-// the loads of a batch never wait for one another.  (i, k) advance incrementally: no
-// division in the loop.
-template <int VEC>
-struct RedVec { typedef float type; };
-template <>
-struct RedVec<4> { typedef float4_t type; };
-
-// VEC consecutive outputs m .. m + VEC - 1 per thread (VEC = 4: one 16-byte load per partial)
-template <int VEC>
-__device__ __forceinline__ typename RedVec<VEC>::type slice_sum_any(const RedMat &r, int T, int t, int m, int ks, const int *nks) {
-    typedef typename RedVec<VEC>::type vec_t;
-    const int total = r.I * r.kmax;
-    const int64_t stride = (int64_t)T * r.M;
-    const float *base = r.part + (int64_t)t * r.M + m;
-    vec_t acc = vec_t(0.f);
-    int i = ks / r.kmax, k = ks - i * r.kmax;                  // slot ks
-    for (int s0 = ks; s0 < total; s0 += RED_BATCH * RED_SL) {
-        vec_t v[RED_BATCH];
-        bool ok[RED_BATCH];
-#pragma unroll
-        for (int j = 0; j < RED_BATCH; j++) {
-            const bool in = s0 + j * RED_SL < total;
-            const int ic = in ? i : 0, kc = in ? k : 0;
-            ok[j] = in && kc < nks[ic];
-            v[j] = *reinterpret_cast<const vec_t *>(base + (int64_t)(ic * r.kmax + kc) * stride);
-            k += RED_SL;
-            while (k >= r.kmax) { k -= r.kmax; i++; }
-        }
-#pragma unroll
-        for (int j = 0; j < RED_BATCH; j++) acc += ok[j] ? v[j] : vec_t(0.f);
-    }
-    return acc;
-}
-
-// nks[i] = workgroups whose unit range touched (block i, row tile rt) of this matrix
-__device__ __forceinline__ void count_partials(const RedMat &r, int rt, int n_chunks, int *nks) {
-    const int nch = n_chunks >> r.pair;
-    for (int i = threadIdx.x; i < r.I; i += RED_OUT * RED_SL) {
-        const int first = (i * r.row_tiles + rt) * nch;
-        nks[i] = (r.sp.owner(first + nch - 1) - r.sp.owner(first) + 1) << r.pair;
-    }
-}
-
-__device__ __forceinline__ float vec_get(float v, int) { return v; }
-__device__ __forceinline__ float vec_get(const float4_t &v, int e) { return v[e]; }
-
-// A workgroup produces RED_OUT * VEC consecutive outputs of one token.  VEC = 4 needs every M a
-// multiple of 4 (16-byte partial loads; the outputs are still stored one by one).
-template <int VEC>
-__global__ __launch_bounds__(RED_OUT * RED_SL) void gemv_reduce_kernel(
-    const RedGroup grp, const half_t *__restrict__ residual, half_t *__restrict__ y, int T, int ldy,
-    int rows_per_tile, int n_chunks) {
-    typedef typename RedVec<VEC>::type vec_t;
-    constexpr int RUN = RED_OUT * VEC;           // outputs per workgroup
-    __shared__ vec_t red[2][RED_SL][RED_OUT];
-    __shared__ int nks[2][RED_MAXBLOCKS];
-    const int lo = threadIdx.x % RED_OUT, ks = threadIdx.x / RED_OUT;
-    int j = 0;
-    if (grp.mode != EPI_SWIGLU) {
-#pragma unroll
-        for (int q = 1; q < GEMV_MAX_GROUP; q++)
-            if (q < grp.n && (int)blockIdx.x >= grp.m[q].first_block) j = q;
-    }
-    const RedMat &r = grp.m[j];
-    // outputs are enumerated per token in runs of RUN rows, so a workgroup never straddles tokens
-    const int local = blockIdx.x - r.first_block;
-    const int per_t = (r.M + RUN - 1) / RUN;
-    const int t = local / per_t, m0 = (local - t * per_t) * RUN, m = m0 + VEC * lo;
-    const int rt = m0 / rows_per_tile;           // RUN divides the tile height
-    const bool live = m < r.M;                   // M % VEC == 0: all VEC outputs or none
-    const bool two = grp.mode == EPI_SWIGLU;
-    count_partials(r, rt, n_chunks, nks[0]);
-    if (two) count_partials(grp.m[1], rt, n_chunks, nks[1]);
-    // residual and bias do not depend on the sums: fetch them before the reduction
-    float extra[VEC], res[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; e++) { extra[e] = 0.f; res[e] = 0.f; }
-    if (ks == 0 && live) {
-#pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            if (r.bias) extra[e] = (float)r.bias[m + e];
-            if (grp.mode == EPI_RESIDUAL) res[e] = (float)residual[(int64_t)t * ldy + r.y_off + m + e];
-        }
-    }
-    float scale = 1.f;
-    __shared__ float ssq[RED_OUT * RED_SL / 64];
-    const bool scaled = grp.xin || grp.ssq;
-    if (scaled) {                                // sum of squares of this token's input row, every workgroup for itself
-        float q = 0.f;
-        if (grp.ssq) {
-            for (int c = threadIdx.x; c < grp.ssq_n; c += RED_OUT * RED_SL) q += grp.ssq[c * T + t];
-        } else {
-            const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
-            for (int c = threadIdx.x * 8; c < grp.n_in; c += RED_OUT * RED_SL * 8) {
-                const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
-#pragma unroll
-                for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
-            }
-        }
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o, 64);
-        if ((threadIdx.x & 63) == 0) ssq[threadIdx.x >> 6] = q;
-    }
-    __syncthreads();
-    if (scaled) {
-        float q = 0.f;
-#pragma unroll
-        for (int w = 0; w < RED_OUT * RED_SL / 64; w++) q += ssq[w];
-        scale = rsqrtf(q / (float)grp.n_in + grp.eps);
-    }
-    red[0][ks][lo] = live ? slice_sum_any<VEC>(r, T, t, m, ks, nks[0]) : vec_t(0.f);
-    if (two) red[1][ks][lo] = live ? slice_sum_any<VEC>(grp.m[1], T, t, m, ks, nks[1]) : vec_t(0.f);
-    __syncthreads();
-    if (ks != 0 || !live) return;
-    vec_t s0 = vec_t(0.f), s1 = vec_t(0.f);
-#pragma unroll
-    for (int k = 0; k < RED_SL; k++) s0 += red[0][k][lo];
-    if (two) {
-#pragma unroll
-        for (int k = 0; k < RED_SL; k++) s1 += red[1][k][lo];
-    }
-#pragma unroll
-    for (int e = 0; e < VEC; e++) {
-        const float a0 = vec_get(s0, e) * scale + extra[e];
-        if (two) {
-            const float a1 = vec_get(s1, e) * scale + (grp.m[1].bias ? (float)grp.m[1].bias[m + e] : 0.f);
-            const float gate = (float)(half_t)a0, up = (float)(half_t)a1;
-            const half_t act = (half_t)(gate / (1.f + __expf(-gate)));
-            y[(int64_t)t * ldy + m + e] = (half_t)((float)act * up);
-        } else {
-            half_t v = (half_t)a0;
-            if (grp.mode == EPI_RESIDUAL) v = (half_t)(res[e] + (float)v);
-            y[(int64_t)t * ldy + r.y_off + m + e] = v;
-        }
-    }
-}
-
-// The same sums for the decode kernels' partials, where EVERY slot of a row holds a number (live
-// partials, zeros in the slots nobody needed): no slot counts, no divisions, and the loads of a thread
-// depend on nothing but its index, so the kernel is one memory round trip long.  A workgroup produces
-// 256 / SL consecutive outputs of one token; SL threads per output take every SL-th of the I * kmax
-// slots (SL = 1: no LDS, no barrier).  SCALED: the input RMS scale of RedGroup::xin.
+// No slot counts, no divisions, and the loads of a thread depend on nothing but its index, so the
+// kernel is one memory round trip long.  A workgroup produces 256 / SL consecutive outputs of one
+// token; SL threads per output take every SL-th of the I * kmax slots (SL = 1: no LDS, no barrier).
+// SCALED: the input RMS scale of RedGroup::xin or RedGroup::ssq.
 constexpr int FLAT_BATCH = 8;
 template <int SL>
 __device__ __forceinline__ float flat_slice_sum(const RedMat &r, int T, int t, int m, int ks) {
@@ -639,11 +491,15 @@ __global__ __launch_bounds__(256) void gemv_reduce_flat_kernel(
     float scale = 1.f;
     if (SCALED) {
         float q = 0.f;
-        const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
-        for (int c = threadIdx.x * 8; c < grp.n_in; c += 256 * 8) {
-            const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
+        if (grp.ssq) {                           // sums of squares per strip group, left by the strip kernel
+            for (int c = threadIdx.x; c < grp.ssq_n; c += 256) q += grp.ssq[c * T + t];
+        } else {
+            const half_t *xr = grp.xin + (int64_t)t * grp.n_in;
+            for (int c = threadIdx.x * 8; c < grp.n_in; c += 256 * 8) {
+                const half8_t v = *reinterpret_cast<const half8_t *>(xr + c);
 #pragma unroll
-            for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+                for (int e = 0; e < 8; e++) q += (float)v[e] * (float)v[e];
+            }
         }
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) q += __shfl_xor(q, o, 64);
@@ -681,7 +537,7 @@ __global__ __launch_bounds__(256) void gemv_reduce_flat_kernel(
 
 template <int SL>
 void launch_reduce_flat(int blocks, const RedGroup &r, const half_t *residual, half_t *y, int T, int ldy, hipStream_t s) {
-    if (r.xin)
+    if (r.xin || r.ssq)
         gemv_reduce_flat_kernel<SL, true><<<blocks, 256, 0, s>>>(r, residual, y, T, ldy);
     else
         gemv_reduce_flat_kernel<SL, false><<<blocks, 256, 0, s>>>(r, residual, y, T, ldy);
@@ -961,21 +817,20 @@ int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T
     r.n_in = N;
     r.eps = eps;
     float *parts[GEMV_MAX_GROUP];
-    // many outputs (tokens x rows) and every M a multiple of 4: four outputs per thread
-    bool vec4 = true;
-    int64_t outputs = 0;
+    // threads per output of the summing kernel, as behind the decode kernels (the strip groups are its slots)
+    int slots = 0;
     for (int j = 0; j < a.n; j++) {
-        vec4 = vec4 && a.M[j] % 4 == 0;
-        outputs += (int64_t)T * a.M[j];
+        const int groups = bs_strip_partials(a.I[j], a.M[j], N, K, T);
+        if (groups > slots) slots = groups;
     }
-    vec4 = vec4 && outputs >= 32768;
-    const int run = vec4 ? 4 * RED_OUT : RED_OUT;
+    const int sl = slots <= FLAT_BATCH ? 1 : slots <= 2 * FLAT_BATCH ? 2 : slots <= 4 * FLAT_BATCH ? 4 : 8;
+    const int run = 256 / sl;
     int ldy = 0, blocks = 0;
     int64_t off = 0;
     for (int j = 0; j < a.n; j++) {
         const int groups = bs_strip_partials(a.I[j], a.M[j], N, K, T);
         parts[j] = part + off;
-        r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], (int)bs_cdiv(a.M[j], run), 1, ldy, blocks, Split{1, 0}};
+        r.m[j] = RedMat{part + off, a.bias[j], groups, a.M[j], 1, ldy, blocks};
         off += (int64_t)groups * T * a.M[j];
         ldy += a.M[j];
         if (mode != EPI_SWIGLU || j == 0) blocks += T * (int)bs_cdiv(a.M[j], run);
@@ -987,10 +842,12 @@ int launch_group_strips(const GroupArgs &a, int N, int K, const half_t *x, int T
     if (st != BS_OK) return st;
     if (mode == EPI_SWIGLU) ldy = a.M[0];
     for (int j = a.n; j < GEMV_MAX_GROUP; j++) r.m[j] = r.m[0];
-    if (vec4)
-        gemv_reduce_kernel<4><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, run, 1);
-    else
-        gemv_reduce_kernel<1><<<blocks, RED_OUT * RED_SL, 0, s>>>(r, residual, y, T, ldy, run, 1);
+    switch (sl) {
+        case 1: launch_reduce_flat<1>(blocks, r, residual, y, T, ldy, s); break;
+        case 2: launch_reduce_flat<2>(blocks, r, residual, y, T, ldy, s); break;
+        case 4: launch_reduce_flat<4>(blocks, r, residual, y, T, ldy, s); break;
+        default: launch_reduce_flat<8>(blocks, r, residual, y, T, ldy, s); break;
+    }
     BS_LAUNCH_CHECK();
     return BS_OK;
 }
@@ -1044,8 +901,7 @@ int launch_group(const GroupArgs &a, int N, int K, const half_t *x, int T, int m
         for (int j = 0; j < a.n; j++) {
             g.m[j] = GemvMat{a.packed[j], a.u[j], a.vt[j], part + p.part_off[j], a.M[j], p.row_tiles[j], p.kmax[j],
                              p.first_wg[j], p.sp[j], p.pair};
-            r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.row_tiles[j], p.kmax[j], y_off, blocks,
-                            p.sp[j], p.pair};
+            r.m[j] = RedMat{part + p.part_off[j], a.bias[j], a.I[j], a.M[j], p.kmax[j], y_off, blocks};
             y_off += a.M[j];
             if (mode != EPI_SWIGLU || j == 0) blocks += tn * (int)bs_cdiv(a.M[j], run);
         }
