@@ -60,6 +60,8 @@ constexpr int NSETS = 3;
 // vb: this lane's fragment of the block's vt image.  All eight fragments and all eight sign vectors are
 // requested first, and every product runs one patch ahead of the FMAs that use it: neither the LDS nor the
 // MFMA latency sits in front of them.
+// FIRST: the sums start here (a zero addend; a plain product would not become a mixed-precision instruction).
+template <bool FIRST>
 __device__ __forceinline__ void rebuild_block(const half_t *vb, const half4_t b, const uint4_t sw, const SignTable st,
                                               float4_t (&acc)[8]) {
     half4_t a[8], sv[8];
@@ -80,7 +82,7 @@ __device__ __forceinline__ void rebuild_block(const half_t *vb, const half4_t b,
         if (s + 1 < 8) p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
         if (s % 2 == 0 && s < 6) lookup(s / 2 + 1);   // the sign vectors of the next two patches, while these two are used
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[s][j] = __builtin_fmaf(p[j], (float)sv[s][j], acc[s][j]);
+        for (int j = 0; j < 4; j++) acc[s][j] = __builtin_fmaf(p[j], (float)sv[s][j], FIRST ? 0.f : acc[s][j]);
     }
 }
 
@@ -190,6 +192,9 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
     // which left the waves waiting for data half of their time.
     // (three token tiles leave registers for two sets only)
     constexpr int NS = TT >= 3 ? 2 : NSETS;
+    // One token tile at rank 16 has the registers for both code versions of a block: the first block of a strip starts
+    // the sums (rebuild_block<true>) instead of adding to accumulators cleared behind the second product.
+    constexpr bool PEEL = TT == 1 && K16;
     half4_t b_set[NS];
     uint4_t sw_set[NS];
 #pragma unroll
@@ -273,7 +278,11 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
     for (int s = 0; s < 8; s++) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
     int i = 0, q = 0, m0 = first_row;
     auto consume = [&](const half4_t &b, const uint4_t &sw) {
-        rebuild_block(vl + (q * I + i) * VBLOCK + aoff, b, sw, st, acc);
+        const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
+        if (PEEL && i == 0)
+            rebuild_block<true>(vb, b, sw, st, acc);
+        else
+            rebuild_block<false>(vb, b, sw, st, acc);
         if (++i < I) return;
         i = 0;
         // y[token, row] of this strip: D[token 4g + v, row lm] = sum_k x[token, col(k)] * w[row, col(k)]
@@ -281,7 +290,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void strip_forward_kernel(
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-            acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            if (!PEEL) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int tt = 0; tt < TT; tt++) {
                 const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
@@ -332,6 +341,7 @@ struct WideMat {
 template <int TT, bool K16>
 __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, const half_t *__restrict__ x, int N, int K, int T) {
     constexpr int WAVES = 8, NT = 64 * WAVES, RS = 16 * WAVES;
+    constexpr bool PEEL = false;                    // (no registers left for the two code versions of a block)
     extern __shared__ __attribute__((aligned(128))) half_t lds_all[];
     half_t *const lds = lds_all + SIGN_LUT_HALVES;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -439,7 +449,11 @@ __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, c
     // the pair being consumed: strip q of the current chunk, block i
     int i = 0, q = 0;
     auto consume = [&](const half4_t &b, const uint4_t &sw) {
-        rebuild_block(vl + (q * I + i) * VBLOCK + aoff, b, sw, st, acc);
+        const half_t *vb = vl + (q * I + i) * VBLOCK + aoff;
+        if (PEEL && i == 0)
+            rebuild_block<true>(vb, b, sw, st, acc);
+        else
+            rebuild_block<false>(vb, b, sw, st, acc);
         if (++i < I) return;
         i = 0;
         // y[token, row] += x[token, these columns] . w[row, these columns], w rounded to fp16 as the dense path rounds it
@@ -447,7 +461,7 @@ __global__ __launch_bounds__(512, 4) void strip_wide_kernel(const WideMat mat, c
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             const half4_t wf = {(half_t)acc[s][0], (half_t)acc[s][1], (half_t)acc[s][2], (half_t)acc[s][3]};
-            acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            if (!PEEL) acc[s] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int tt = 0; tt < TT; tt++) {
                 const half4_t xf = *reinterpret_cast<const half4_t *>(xq + tt * 16 * xstride + 32 * (s >> 1) + 4 * (s & 1));
