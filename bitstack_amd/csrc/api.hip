@@ -14,6 +14,7 @@ extern "C" const char *bs_error_string(int status) {
         case BS_ERR_ALIGN: return "pointer is not aligned as the entry point requires";
         case BS_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case BS_ERR_NO_DEVICE: return "no usable HIP device";
+        case BS_ERR_LIBRARY: return "the vendor GEMM library failed after it had accepted the call";
         default: break;
     }
     if (status <= BS_ERR_HIP_BASE) return hipGetErrorString((hipError_t)(BS_ERR_HIP_BASE - status));
@@ -29,21 +30,14 @@ static int forward_dims(int I, int M, int N, int K, int T) {
 
 static int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
-// Which kernel multiplies the rebuilt weight: 0 by token count, 1 always linear_f16_kernel, 2 hipBLASLt
-// wherever it takes the shape (bs_set_dense_kernel, for tests and benchmarks).
-static int g_dense_kernel = 0;
-// From this many tokens on the library's kernels are the faster ones behind the rebuild on the layer shapes measured
-// (1024 x 4096 .. 14336 x 4096 with 8 blocks, rebuild included, the four layers run in turn so that no layer finds its
-// operands in cache; microseconds over the four, linear_f16_kernel / library): 64 tokens 256-268 / 243-247 (only
-// 14336 x 4096 rebuilds there), 128 tokens 326-336 / 304-307, 256 tokens 325-344 / 312-314, 448 tokens 397-409 /
-// 373-374, 2048 tokens 662 / 840 useful TFLOP/s.  The library's choice of kernel is poor at a few token counts (160 and
-// 192 tokens on 4096 x 14336: 144-154 against 130-139), where the sums come out level.  Below, no shape measured
-// rebuilds a weight that the strip kernels would not take, and linear_f16_kernel's small tiles serve.
-constexpr int DENSE_LIBRARY_MIN_T = 49;
+// Which kernel multiplies the rebuilt weight: this library's linear_f16_kernel unless the calling thread has asked
+// for hipBLASLt with bs_set_dense_kernel(BS_DENSE_LIBRARY) (a comparator for tests and benchmarks: what the
+// reference's F.linear runs on ROCm).  The setting belongs to the thread that made it, so a size query and the
+// forward that follows it on the same thread always agree, whatever other threads do.
+static thread_local int g_dense_kernel = 0;
 
-static bool dense_wants_library(int M, int N, int T) {
-    if (g_dense_kernel == BS_DENSE_OWN || M % 8 != 0 || N % 8 != 0) return false;
-    return g_dense_kernel == BS_DENSE_LIBRARY || T >= DENSE_LIBRARY_MIN_T;
+static bool dense_wants_library(int M, int N) {
+    return g_dense_kernel == BS_DENSE_LIBRARY && M % 8 == 0 && N % 8 == 0;
 }
 
 extern "C" int bs_set_dense_kernel(int mode) {
@@ -60,7 +54,7 @@ static int64_t workspace_need(int I, int M, int N, int K, int T, bool library_ok
     int64_t gemv = bs_gemv_workspace_bytes(I, M, N, K, T);
     if (gemv > 0) return round_up(gemv, 256);
     // the rebuilt weight, then the library GEMM's own scratch where that is the kernel
-    return round_up((int64_t)M * N * 2, 256) + (library_ok && dense_wants_library(M, N, T) ? BS_DENSE_LIBRARY_WORKSPACE : 0);
+    return round_up((int64_t)M * N * 2, 256) + (library_ok && dense_wants_library(M, N) ? BS_DENSE_LIBRARY_WORKSPACE : 0);
 }
 
 extern "C" int64_t bs_workspace_bytes(int I, int M, int N, int K, int T) { return workspace_need(I, M, N, K, T, true); }
@@ -106,10 +100,10 @@ static int forward_impl(const uint8_t *packed, const void *u, const void *vt, co
     half_t *w = (half_t *)workspace;
     st = bs_launch_reconstruct_packed(packed, (const half_t *)u, (const half_t *)vt, w, I, M, N, K, s);
     if (st != BS_OK) return st;
-    if (library_ok && dense_wants_library(M, N, T)) {
+    if (library_ok && dense_wants_library(M, N)) {
         st = bs_launch_linear_library((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N,
                                       (char *)workspace + round_up((int64_t)M * N * 2, 256), s);
-        if (st != BS_ERR_SHAPE) return st;      // enqueued, or failed for good; BS_ERR_SHAPE: not for this call
+        if (st != BS_ERR_SHAPE) return st;      // enqueued, or failed for good; BS_ERR_SHAPE: declined before anything was enqueued
     }
     return bs_launch_linear_f16((const half_t *)x, w, (const half_t *)bias, (half_t *)y, T, M, N, s);
 }
@@ -151,8 +145,8 @@ extern "C" int bs_forward_static(const uint8_t *packed, const void *u, const voi
     if (st != BS_OK) return st;
     if (T == 0) return BS_OK;
     // sizes first: a call that would not fit is refused before any device is touched.  The dense product
-    // always runs this library's own kernel here: the vendor GEMM wants 64 MiB of scratch of its own, and
-    // setting it up allocates.
+    // always runs this library's own kernel here, whatever bs_set_dense_kernel says: the vendor GEMM wants
+    // 64 MiB of scratch of its own, and setting it up allocates.
     const int64_t need = workspace_need(I, M, N, K, T, false);
     if (need < 0) return (int)need;
     if (need > (int64_t)BS_STATIC_SCRATCH_BYTES) return BS_ERR_WORKSPACE;

@@ -1,12 +1,12 @@
-// The dense product y[T, M] = x[T, N] @ w[M, N]^T (+ bias) through hipBLASLt, for the token counts
-// where the library's tuned kernels beat linear_f16_kernel (gemm.hip).  After the weight has been
-// rebuilt this is a plain fp16 GEMM with fp32 accumulation, the product the reference hands to
-// F.linear (bitstack/modules/BitStackLinear.py:132,140,148) - which on ROCm is this library.
+// The dense product y[T, M] = x[T, N] @ w[M, N]^T (+ bias) through hipBLASLt: a COMPARATOR for tests
+// and benchmarks, never chosen by bs_forward on its own (bs_set_dense_kernel(BS_DENSE_LIBRARY) asks for
+// it per thread).  After the weight has been rebuilt the product is a plain fp16 GEMM with fp32
+// accumulation, what the reference hands to F.linear (bitstack/modules/BitStackLinear.py:132,140,148)
+// - which on ROCm is this library - so it is the yardstick linear_f16_kernel (gemm.hip) is timed against.
 //
 // hipBLASLt is opened at run time (dlopen of its SONAME), so libbitstack_hip.so has no link-time
-// dependency on it: where it is missing, or refuses a shape, the caller falls back to its own
-// kernel.  In a process that already holds a copy (PyTorch ships one under the same SONAME) that
-// copy is the one used.
+// dependency on it.  In a process that already holds a copy (PyTorch ships one under the same SONAME)
+// that copy is the one used.
 //
 // Row-major operands read as column-major ones: w is A = [N x M] (ld N, transposed), x is
 // B = [N x T] (ld N), y is D = [M x T] (ld M); D = A^T B, bias broadcast along D's rows.
@@ -24,7 +24,9 @@ namespace {
 struct LtApi {
     decltype(&hipblasLtCreate) create;
     decltype(&hipblasLtMatrixLayoutCreate) layout_create;
+    decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy;
     decltype(&hipblasLtMatmulDescCreate) desc_create;
+    decltype(&hipblasLtMatmulDescDestroy) desc_destroy;
     decltype(&hipblasLtMatmulDescSetAttribute) desc_set;
     decltype(&hipblasLtMatmulPreferenceCreate) pref_create;
     decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set;
@@ -33,8 +35,7 @@ struct LtApi {
     decltype(&hipblasLtMatmul) matmul;
 };
 
-// One descriptor set and one chosen algorithm per (device, T, M, N, bias?); kept until the process
-// ends (a few hundred bytes of host memory each).
+// One descriptor set and one chosen algorithm per (device, T, M, N, bias?).
 struct LtPlan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t a = nullptr, b = nullptr, d = nullptr;
@@ -42,6 +43,12 @@ struct LtPlan {
     size_t workspace = 0;
     bool usable = false;
 };
+
+// The plan table is bounded: a caller that sweeps prompt lengths would otherwise add an entry (and a
+// heuristic query) per distinct token count for the life of the process.  When it is full it is emptied
+// and rebuilt on demand - but only outside stream capture, where no graph can be recording the
+// descriptors (a descriptor only lives on the host; recorded launches hold none of it).
+constexpr size_t LT_MAX_PLANS = 256;
 
 struct LtState {
     std::mutex mu;                    // one caller at a time: the bias pointer is an attribute of the shared descriptor
@@ -66,7 +73,9 @@ bool load_api(LtState &st) {
     if (!so) return false;
     LtApi &a = st.api;
     st.loaded = resolve(so, "hipblasLtCreate", a.create) && resolve(so, "hipblasLtMatrixLayoutCreate", a.layout_create) &&
+                resolve(so, "hipblasLtMatrixLayoutDestroy", a.layout_destroy) &&
                 resolve(so, "hipblasLtMatmulDescCreate", a.desc_create) &&
+                resolve(so, "hipblasLtMatmulDescDestroy", a.desc_destroy) &&
                 resolve(so, "hipblasLtMatmulDescSetAttribute", a.desc_set) &&
                 resolve(so, "hipblasLtMatmulPreferenceCreate", a.pref_create) &&
                 resolve(so, "hipblasLtMatmulPreferenceSetAttribute", a.pref_set) &&
@@ -75,7 +84,15 @@ bool load_api(LtState &st) {
     return st.loaded;
 }
 
-bool make_plan(LtState &st, hipblasLtHandle_t h, LtPlan &p, int T, int M, int N, bool bias) {
+void destroy_plan(const LtApi &a, LtPlan &p) {
+    if (p.a) a.layout_destroy(p.a);
+    if (p.b) a.layout_destroy(p.b);
+    if (p.d) a.layout_destroy(p.d);
+    if (p.desc) a.desc_destroy(p.desc);
+    p = LtPlan{};
+}
+
+bool fill_plan(LtState &st, hipblasLtHandle_t h, LtPlan &p, int T, int M, int N, bool bias) {
     const LtApi &a = st.api;
     const auto ok = [](hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; };
     if (!ok(a.desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F))) return false;
@@ -114,14 +131,23 @@ bool make_plan(LtState &st, hipblasLtHandle_t h, LtPlan &p, int T, int M, int N,
     return found;
 }
 
+// A plan that cannot be completed leaves nothing behind but the (empty) table entry that says so.
+void make_plan(LtState &st, hipblasLtHandle_t h, LtPlan &p, int T, int M, int N, bool bias) {
+    if (fill_plan(st, h, p, T, M, N, bias)) {
+        p.usable = true;
+    } else {
+        destroy_plan(st.api, p);
+    }
+}
+
 }  // namespace
 
-// BS_OK when the product has been enqueued; BS_ERR_SHAPE when hipBLASLt is not available or has no
-// kernel for the shape (the caller then runs its own).  `workspace` holds BS_DENSE_LIBRARY_WORKSPACE
-// bytes, 256-byte aligned.  The first call for a shape on a device creates the library's handle and
-// asks its heuristic (host work, and the library may allocate); a shape first seen while its stream is
-// being captured is therefore declined (BS_ERR_SHAPE), and only shapes already run once eagerly are
-// recorded into a graph.
+// BS_OK: the product has been enqueued.  BS_ERR_SHAPE: declined BEFORE anything was enqueued - hipBLASLt is
+// not installed, has no kernel for the shape, the buffers are not aligned for it, or the shape is new
+// while its stream is being captured (setting the library up is host work that may allocate) - and the
+// caller runs its own kernel.  Anything else is a failure after the call had been accepted (a HIP
+// status, or BS_ERR_LIBRARY for a hipBLASLt one): final, the caller must not paper over it.
+// `workspace` holds BS_DENSE_LIBRARY_WORKSPACE bytes, 256-byte aligned.
 int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bias, half_t *y, int T, int M, int N,
                              void *workspace, hipStream_t s) {
     if (!bs_aligned(x, 16) || !bs_aligned(w, 16) || !bs_aligned(y, 16) || N % 8 != 0 || M % 8 != 0) return BS_ERR_SHAPE;
@@ -133,17 +159,20 @@ int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bia
     const auto key = std::make_tuple(dev, T, M, N, bias ? 1 : 0);
     auto it = st.plans.find(key);
     if (it == st.plans.end()) {
-        // Setting the library up (loading it, its handle, the heuristic) is host work that may allocate:
-        // never under stream capture.  A shape first seen while capturing runs the caller's own kernel.
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return BS_ERR_SHAPE;
+        BS_HIP_TRY(hipStreamIsCapturing(s, &cap));
+        if (cap != hipStreamCaptureStatusNone) return BS_ERR_SHAPE;
         if (!load_api(st)) return BS_ERR_SHAPE;
         if (!st.handle[dev] && st.api.create(&st.handle[dev]) != HIPBLAS_STATUS_SUCCESS) {
             st.handle[dev] = nullptr;
             return BS_ERR_SHAPE;
         }
+        if (st.plans.size() >= LT_MAX_PLANS) {
+            for (auto &kv : st.plans) destroy_plan(st.api, kv.second);
+            st.plans.clear();
+        }
         LtPlan p;
-        p.usable = make_plan(st, st.handle[dev], p, T, M, N, bias != nullptr);
+        make_plan(st, st.handle[dev], p, T, M, N, bias != nullptr);
         it = st.plans.emplace(key, p).first;
     }
     LtPlan &p = it->second;
@@ -151,10 +180,10 @@ int bs_launch_linear_library(const half_t *x, const half_t *w, const half_t *bia
     if (bias) {
         const void *bp = bias;
         if (st.api.desc_set(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp)) != HIPBLAS_STATUS_SUCCESS)
-            return BS_ERR_SHAPE;
+            return BS_ERR_LIBRARY;
     }
     const float alpha = 1.f, beta = 0.f;
     const hipblasStatus_t r = st.api.matmul(st.handle[dev], p.desc, &alpha, w, p.a, x, p.b, &beta, y, p.d, y, p.d, &p.algo,
                                             workspace, p.workspace, s);
-    return r == HIPBLAS_STATUS_SUCCESS ? BS_OK : BS_ERR_SHAPE;
+    return r == HIPBLAS_STATUS_SUCCESS ? BS_OK : BS_ERR_LIBRARY;
 }

@@ -555,8 +555,9 @@ struct Plan {
 // One instantiation and one grid for the whole group; every matrix gets a share of
 // the workgroups in proportion to its units.
 // Which kernel make_plan picks for one and two tokens: 0 by shape, 1 always the fp16 kernel, 2 the block-scaled one
-// wherever it takes the shape (bs_set_decode_kernel, for tests and benchmarks).
-int g_decode_kernel = 0;
+// wherever it takes the shape (bs_set_decode_kernel, for tests and benchmarks).  Per calling thread: a size query
+// and the forward behind it on one thread agree whatever other threads set.
+thread_local int g_decode_kernel = 0;
 
 // Rows per workgroup of the block-scaled kernel for these matrices (0: it does not run them).
 int mx_rows_per_tile(const int *I, const int *M, int n, int N, int K, int T) {

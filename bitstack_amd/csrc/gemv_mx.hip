@@ -54,6 +54,7 @@ namespace {
 typedef int v8i_t __attribute__((ext_vector_type(8)));
 typedef unsigned v6u_t __attribute__((ext_vector_type(6)));
 typedef _Float16 half32_t __attribute__((ext_vector_type(32)));
+typedef uint16_t ushort2_t __attribute__((ext_vector_type(2)));
 
 constexpr int MX_WAVES = 8;
 constexpr int MX_OPERAND = 64 * 16 + 64 * 8;        // bytes of one (half, q, term) operand: dwords 0-3, then dwords 4-5, per lane
@@ -106,20 +107,27 @@ __device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, c
 #pragma unroll
     for (int e = 0; e < 4; e++) zw[e] = *reinterpret_cast<const uint4_t *>(stage + ((k * 4 + q) * 4 + g) * MX_STAGE_BLK + 4 * e);
     half32_t z;
-    half2_t mx = {(half_t)0, (half_t)0};
+    // Block maximum of |z| on the BIT PATTERNS (unsigned 16-bit compare: monotonic for magnitudes, and
+    // Inf = 0x7C00 < every NaN), so a NaN or an infinity in vt * x is seen instead of being dropped the way
+    // a floating-point max drops NaN.  fp6 has no encoding for either: a block that holds one gets the
+    // E8M0 scale 0xFF (NaN) on all three terms, every product of the block is NaN, and so is every output
+    // that the column contributes to - as F.linear, and the fp16 kernel, give a non-finite result there.
+    ushort2_t mxb = {0, 0};
 #pragma unroll
     for (int b = 0; b < 16; b++) {
         const uint32_t word = zw[b >> 2][b & 3];      // (a bit cast applied to the element expression itself reads element 0)
         const half2_t v = __builtin_bit_cast(half2_t, word);
         z[2 * b] = v[0];
         z[2 * b + 1] = v[1];
-        mx = __builtin_elementwise_max(mx, __builtin_elementwise_abs(v));
+        mxb = __builtin_elementwise_max(mxb, __builtin_bit_cast(ushort2_t, word & 0x7FFF7FFFu));
     }
-    const float m = fmaxf((float)mx[0], (float)mx[1]);
+    const uint16_t mbits = mxb[0] > mxb[1] ? mxb[0] : mxb[1];
+    const bool finite = mbits < 0x7C00u;
+    const float m = (float)__builtin_bit_cast(half_t, mbits);
     // exponent of s1 = floor(log2(m * 16 / 15)) - 2: the conversions use the exponent only
-    const float s1 = fmaxf(m * (4.f / 15.f), 0x1p-100f), s2 = s1 * 0x1p-4f, s3 = s1 * 0x1p-8f;
+    const float s1 = finite ? fmaxf(m * (4.f / 15.f), 0x1p-100f) : 1.f, s2 = s1 * 0x1p-4f, s3 = s1 * 0x1p-8f;
     const uint32_t e1 = __builtin_bit_cast(uint32_t, s1) >> 23;
-    const uint32_t scale = e1 | ((e1 - 4u) << 8) | ((e1 - 8u) << 16);
+    const uint32_t scale = finite ? (e1 | ((e1 - 4u) << 8) | ((e1 - 8u) << 16)) : 0x00FFFFFFu;
     const v6u_t t1 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(z, s1);
     const half32_t r1 = z - __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t1, s1);
     const v6u_t t2 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(r1, s2);

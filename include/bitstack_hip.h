@@ -37,6 +37,7 @@ extern "C" {
 #define BS_ERR_ALIGN         -4   /* pointer not aligned as documented               */
 #define BS_ERR_WORKSPACE     -5   /* workspace missing or smaller than required      */
 #define BS_ERR_NO_DEVICE     -6   /* no HIP device / wrong architecture              */
+#define BS_ERR_LIBRARY       -7   /* the vendor GEMM (comparator mode only) failed   */
 #define BS_ERR_HIP_BASE   -1000   /* -(1000 + hipError_t) for a failed HIP call      */
 
 /* Library version, major * 10000 + minor * 100 + patch. */
@@ -116,8 +117,8 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * hipMalloc).  No counterpart in the reference.  The scratch of the kernels is a
  * device array inside the library, BS_STATIC_SCRATCH_BYTES per GPU, held until
  * the process ends; the call allocates nothing and frees nothing.  Dimensions
- * whose scratch (bs_workspace_bytes, less the vendor GEMM's 64 MiB where
- * bs_forward would use it) exceeds BS_STATIC_SCRATCH_BYTES return
+ * whose scratch (bs_workspace_bytes in the default dense-kernel mode) exceeds
+ * BS_STATIC_SCRATCH_BYTES return
  * BS_ERR_WORKSPACE: 64 MiB holds the partial sums of every 1..4-token forward of
  * the 8B and 70B linear shapes up to 36 blocks and of their 5..8-token forwards
  * up to 12 blocks; the strip kernel at several dozen tokens on the largest
@@ -125,10 +126,14 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * (more than 96 tokens, or N not a multiple of 128) need more and are refused.
  * All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (different streams, different host threads) race; calls on one
- * stream are ordered and safe.  Same results as bs_forward, bit for bit; where
- * a weight is rebuilt, as bs_forward under bs_set_dense_kernel(BS_DENSE_OWN),
- * because the dense product here always runs this library's own kernel (the
- * vendor GEMM needs scratch of its own and allocates when it is set up).
+ * stream are ordered and safe.  Same results as bs_forward, bit for bit, for
+ * the same arguments (the comparator mode of bs_set_dense_kernel is ignored
+ * here: the vendor GEMM needs scratch of its own and allocates when it is set
+ * up).  The FIRST call per device and kernel must be made outside stream
+ * capture: it looks the array's address up and, for kernels with more than
+ * 64 KB of LDS, raises their limit - host-side set-up that a capture does not
+ * record.  The array used is that of the device current at the call, which
+ * must be the device of `stream`.
  */
 #define BS_STATIC_SCRATCH_BYTES (64 << 20)
 int bs_forward_static(const uint8_t *packed, const void *u, const void *vt, const void *x,
@@ -162,27 +167,28 @@ int bs_decode_kernel(int I, int M, int N, int K, int T);
  * Test and benchmark hook: 0 = choose the decode kernel of one- and two-token
  * passes by shape (the default), BS_DECODE_F16 = always the fp16 kernel,
  * BS_DECODE_MX = the block-scaled kernel wherever it takes the shape
- * (N % 512 == 0, at most two tokens).  Process-wide and not synchronised: set it while
- * no other thread is inside the library.  Workspace sizes and bs_decode_plan
- * follow the setting.  No counterpart in the reference.
+ * (N % 512 == 0, at most two tokens).  The setting belongs to the CALLING
+ * THREAD (every thread starts at 0): bs_workspace_bytes, bs_decode_plan and
+ * bs_forward called from one thread always agree, whatever other threads set.
+ * No counterpart in the reference.
  */
 int bs_set_decode_kernel(int mode);
 
 /*
  * Test and benchmark hook: which kernel multiplies the rebuilt weight in
- * bs_forward's large-T path.  0 = by token count (the default: this library's
- * linear_f16 kernels below 49 tokens, hipBLASLt from there on),
- * BS_DENSE_OWN = always this library's kernels, BS_DENSE_LIBRARY = hipBLASLt
- * wherever it takes the shape (M and N multiples of 8).  hipBLASLt is opened
- * at run time; where it is missing or has no kernel for a shape the call runs
- * this library's kernel.  bs_workspace_bytes follows the setting (the library
- * GEMM gets 64 MiB of scratch behind the rebuilt weight).  The first call for
- * a shape sets the library up (host work, possibly allocations); a shape first
- * seen under stream capture runs this library's kernel instead, so run a shape
- * once eagerly if the captured graph is to hold the library GEMM.  Process-wide and not synchronised, like
- * bs_set_decode_kernel.  In the reference this product is F.linear on the
- * rebuilt weight (bitstack/modules/BitStackLinear.py:132,140,148), which on
- * ROCm is the same library.
+ * bs_forward's large-T path.  0 and BS_DENSE_OWN = this library's linear_f16
+ * kernels (the default, and the only kernels bs_forward ever picks by itself),
+ * BS_DENSE_LIBRARY = hipBLASLt wherever it takes the shape (M and N multiples of
+ * 8, 16-byte aligned y): the comparator the own kernels are timed against; in
+ * the reference this product is F.linear on the rebuilt weight
+ * (bitstack/modules/BitStackLinear.py:132,140,148), which on ROCm is that
+ * library.  hipBLASLt is opened at run time; where it is missing, has no kernel
+ * for a shape, or the shape is first seen under stream capture (setting the
+ * library up is host work that may allocate) the call runs this library's
+ * kernel; a failure after the library has accepted the call is returned
+ * (BS_ERR_LIBRARY or a HIP status), not papered over.  In library mode
+ * bs_workspace_bytes adds 64 MiB of scratch for it behind the rebuilt weight.
+ * Per calling thread, like bs_set_decode_kernel.
  */
 #define BS_DENSE_OWN     1
 #define BS_DENSE_LIBRARY 2

@@ -19,7 +19,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not available")
-@pytest.mark.parametrize("src", ["gemv.hip", "gemm.hip", "reconstruct.hip", "strip.hip", "pack.hip", "decode_step.hip"])
+@pytest.mark.parametrize("src", ["gemv.hip", "gemv_mx.hip", "gemm.hip", "reconstruct.hip", "strip.hip", "pack.hip", "decode_step.hip"])
 def test_no_spill_code_in_loops_and_little_scratch(src, tmp_path):
     asm = tmp_path / "k.s"
     out = subprocess.run([HIPCC] + FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", str(asm)],

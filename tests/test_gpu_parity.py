@@ -220,6 +220,37 @@ def test_forward_decode_block_scaled_kernel(I, M, N, K, T, decode_kernel):
     assert_close(y, y16.float().cpu().numpy(), "vs the fp16 decode kernel", 2e-3, 3e-4)
 
 
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
+def test_non_finite_activations_stay_non_finite_on_both_decode_kernels(bad, decode_kernel):
+    """F.linear on the rebuilt weight (bitstack/modules/BitStackLinear.py:114) gives a non-finite y[t, :]
+    for a token whose x holds a NaN or an infinity.  fp6 has no encoding for either, so the block-scaled
+    kernel carries them in the block's scale: every output of that token must come out non-finite on
+    both decode kernels, and the other token of a two-token call must stay as it was."""
+    I, M, N = 3, 1024, 4096
+    q, u, vt, x = synthetic_layer(M, N, I, 2, seed=77, device=dev())
+    clean = {}
+    for T in (1, 2):
+        for col in (0, 777, N - 1):
+            xb = x[:T].clone()
+            xb[0, col] = bad
+            for mode in (_lib.DECODE_F16, _lib.DECODE_MX):
+                decode_kernel(mode)
+                assert _lib.lib().bs_decode_kernel(I, M, N, 16, T) == mode
+                if (T, mode) not in clean:
+                    clean[(T, mode)] = IU.bitstack_forward_hip(q, u, vt, x[:T].contiguous())
+                y = IU.bitstack_forward_hip(q, u, vt, xb)
+                assert not bool(torch.isfinite(y[0]).any()), (T, col, mode)
+                if T == 2:
+                    assert torch.equal(y[1], clean[(T, mode)][1]), (col, mode)
+    # a non-finite weight factor: every token's outputs
+    vb = vt.clone()
+    vb[1, 5, 1234] = bad
+    for mode in (_lib.DECODE_F16, _lib.DECODE_MX):
+        decode_kernel(mode)
+        y = IU.bitstack_forward_hip(q, u, vb, x)
+        assert not bool(torch.isfinite(y).any()), mode
+
+
 def test_block_scaled_kernel_is_declined_where_it_does_not_apply(decode_kernel):
     decode_kernel(_lib.DECODE_MX)
     L = _lib.lib()
@@ -707,8 +738,8 @@ def _random_forced_cases(n, seed):
         kind = rng.integers(0, 5)
         if kind == 0:      # decode kernels, many blocks (long partial-sum lists)
             N = 512 * int(rng.integers(1, 9)); M = int(rng.integers(1, 3000)); T = int(rng.integers(1, 5)); I = int(rng.integers(1, 40))
-        elif kind == 1:    # one and two tokens on wide matrices (several units per workgroup)
-            N = 512 * int(rng.integers(1, 17)); M = 64 * int(rng.integers(1, 120)); T = int(rng.integers(1, 3)); I = int(rng.integers(1, 20))
+        elif kind == 1:    # one and two tokens on wide matrices (several units per workgroup), up to the widest 8B layer
+            N = 512 * int(rng.integers(1, 29)); M = 64 * int(rng.integers(1, 120)); T = int(rng.integers(1, 3)); I = int(rng.integers(1, 20))
         elif kind == 2:    # strip kernel
             N = 128 * int(rng.integers(1, 40)); M = int(rng.integers(1, 2500)); T = int(rng.integers(5, 49)); I = int(rng.integers(1, 12))
         elif kind == 3:    # rebuild + dense, ragged everything

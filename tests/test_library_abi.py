@@ -38,7 +38,7 @@ def test_every_declared_symbol_is_exported(L):
 def test_version_and_error_strings(L):
     assert L.bs_version() >= 100
     assert _lib.error_string(0) == "ok"
-    for code in (-1, -2, -3, -4, -5, -6):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert _lib.error_string(code) not in ("ok", "unknown status")
     assert _lib.error_string(-999) == "unknown status"
 
@@ -76,8 +76,11 @@ def test_workspace_bytes(L):
     assert L.bs_workspace_bytes(8, 4096, 4096, 16, 0) == 0
     assert L.bs_workspace_bytes(8, 4096, 4100, 16, 1) == -2
     assert L.bs_workspace_bytes(8, 4096, 4096, 20, 1) == -3
-    # prefill and odd shapes rebuild the fp16 weight (from 49 tokens followed by 64 MiB for the vendor GEMM)
+    # prefill and odd shapes rebuild the fp16 weight (the vendor GEMM and its 64 MiB only in comparator mode)
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2
+    assert L.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
     assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2 + (64 << 20)
+    assert L.bs_set_dense_kernel(_lib.DENSE_AUTO) == 0
     assert L.bs_workspace_bytes(8, 4096, 4104, 16, 20) == 4096 * 4104 * 2
     assert L.bs_workspace_bytes(2, 64, 72, 16, 1) == ((64 * 72 * 2 + 255) // 256) * 256
     # decode keeps fp32 partial row sums: a multiple of T * M * 4, far below the weight
@@ -88,6 +91,33 @@ def test_workspace_bytes(L):
     for T in (8, 32, 48):
         b = L.bs_workspace_bytes(8, 4096, 4096, 16, T)
         assert T * 4096 * 4 <= b <= 32 * (T * 4096 * 4 + T * 4) + 256
+
+
+def test_kernel_hooks_belong_to_the_calling_thread(L):
+    """A hook set on one thread moves neither the plan nor the workspace size another thread sees."""
+    import threading
+    seen = {}
+
+    def other():
+        seen["decode"] = L.bs_decode_kernel(4, 4096, 4096, 16, 1)
+        seen["ws"] = L.bs_workspace_bytes(4, 4096, 4096, 16, 512)
+        # and what this thread sets stays here
+        L.bs_set_decode_kernel(_lib.DECODE_F16)
+
+    base_decode = L.bs_decode_kernel(4, 4096, 4096, 16, 1)
+    base_ws = L.bs_workspace_bytes(4, 4096, 4096, 16, 512)
+    try:
+        assert L.bs_set_decode_kernel(_lib.DECODE_MX) == 0 and L.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
+        assert L.bs_decode_kernel(4, 4096, 4096, 16, 1) == _lib.DECODE_MX
+        assert L.bs_workspace_bytes(4, 4096, 4096, 16, 512) == base_ws + (64 << 20)
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        assert seen == {"decode": base_decode, "ws": base_ws}
+        assert L.bs_decode_kernel(4, 4096, 4096, 16, 1) == _lib.DECODE_MX
+    finally:
+        L.bs_set_decode_kernel(_lib.DECODE_AUTO)
+        L.bs_set_dense_kernel(_lib.DENSE_AUTO)
 
 
 def test_group_and_decode_step_validation(L):
