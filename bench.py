@@ -60,6 +60,8 @@ def parse():
     ap.add_argument("--tokens", type=int, default=2, help="tokens per forward of --only sweep_tokens (the 20-layer sweep at that count)")
     ap.add_argument("--layer", default="14336x4096x16x1",
                     help="with --only one_layer: out x in x blocks x tokens of the single layer to run (counter runs)")
+    ap.add_argument("--decode-kernel", choices=["auto", "f16", "mx"], default="auto",
+                    help="with --only sweep_tokens / one_layer: force the fp16 or the block-scaled decode kernel (A/B timing)")
     ap.add_argument("--detail", default=None, help="write per-layer timings to this JSON file")
     return ap.parse_args()
 
@@ -373,6 +375,10 @@ def main():
             del lp
         return pre
 
+    if a.only in ("one_layer", "sweep_tokens"):
+        # (the setting is this thread's; the process ends with the measurement)
+        _lib.check(lib.bs_set_decode_kernel({"auto": _lib.DECODE_AUTO, "f16": _lib.DECODE_F16, "mx": _lib.DECODE_MX}[a.decode_kernel]),
+                   "bs_set_decode_kernel")
     if a.only == "one_layer":
         # 12 forwards of ONE layer on 3 rotating copies of its buffers (as every layer of the sweep
         # is run), nothing else on the GPU: the process to put under rocprofv3 --pmc

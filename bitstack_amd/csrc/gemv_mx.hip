@@ -55,11 +55,14 @@ typedef int v8i_t __attribute__((ext_vector_type(8)));
 typedef unsigned v6u_t __attribute__((ext_vector_type(6)));
 typedef _Float16 half32_t __attribute__((ext_vector_type(32)));
 typedef uint16_t ushort2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v16u_t __attribute__((ext_vector_type(16)));
 
 constexpr int MX_WAVES = 8;
 constexpr int MX_OPERAND = 64 * 16 + 64 * 8;        // bytes of one (half, q, term) operand: dwords 0-3, then dwords 4-5, per lane
 constexpr int MX_SCALES = 8 * 3 * MX_OPERAND;       // the scale words of a Z buffer follow its 24 operands
 constexpr int MX_ZBUF = MX_SCALES + 8 * 64 * 4;     // bytes per Z buffer
+
+__device__ __forceinline__ uint32_t mx_and_or(uint32_t w, uint32_t mask, uint32_t base) { return (w & mask) | base; }
 
 __device__ __forceinline__ float4_t mx_mfma(const uint4_t &a03, const uint2_t &a45, const uint4_t &b, float4_t c,
                                             int term, uint32_t scale_a, uint32_t scale_b) {
@@ -84,13 +87,13 @@ constexpr int MX_STAGE_BLK = 20;                     // dwords per staged (rank,
                                                      // 16-byte reads of 8 consecutive lanes hit 8 different bank groups
 constexpr int MX_STAGE = 64 * MX_STAGE_BLK * 4;      // bytes of staging per wave
 __device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, const half8_t (&pv)[4], const half8_t &px,
-                                                  int h, int j, int lane, int K) {
+                                                  int h, int j, int lane) {
     {
         const int g = lane >> 4, b = lane & 15;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            half8_t p = pv[k] * px;
-            if (4 * j + k >= K) p = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
+            // (ranks beyond K carry a copy of rank K - 1: the flush multiplies them by u = 0)
+            const half8_t p = pv[k] * px;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 half2_t pr = {p[7 - q], p[3 - q]};
@@ -106,21 +109,20 @@ __device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, c
     uint4_t zw[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) zw[e] = *reinterpret_cast<const uint4_t *>(stage + ((k * 4 + q) * 4 + g) * MX_STAGE_BLK + 4 * e);
-    half32_t z;
     // Block maximum of |z| on the BIT PATTERNS (unsigned 16-bit compare: monotonic for magnitudes, and
     // Inf = 0x7C00 < every NaN), so a NaN or an infinity in vt * x is seen instead of being dropped the way
     // a floating-point max drops NaN.  fp6 has no encoding for either: a block that holds one gets the
     // E8M0 scale 0xFF (NaN) on all three terms, every product of the block is NaN, and so is every output
     // that the column contributes to - as F.linear, and the fp16 kernel, give a non-finite result there.
+    v16u_t zwords;
     ushort2_t mxb = {0, 0};
 #pragma unroll
     for (int b = 0; b < 16; b++) {
-        const uint32_t word = zw[b >> 2][b & 3];      // (a bit cast applied to the element expression itself reads element 0)
-        const half2_t v = __builtin_bit_cast(half2_t, word);
-        z[2 * b] = v[0];
-        z[2 * b + 1] = v[1];
+        const uint32_t word = zw[b >> 2][b & 3];
+        zwords[b] = word;
         mxb = __builtin_elementwise_max(mxb, __builtin_bit_cast(ushort2_t, word & 0x7FFF7FFFu));
     }
+    const half32_t z = __builtin_bit_cast(half32_t, zwords);
     const uint16_t mbits = mxb[0] > mxb[1] ? mxb[0] : mxb[1];
     const bool finite = mbits < 0x7C00u;
     const float m = (float)__builtin_bit_cast(half_t, mbits);
@@ -128,10 +130,21 @@ __device__ __forceinline__ void mx_produce_finish(char *zbuf, uint32_t *stage, c
     const float s1 = finite ? fmaxf(m * (4.f / 15.f), 0x1p-100f) : 1.f, s2 = s1 * 0x1p-4f, s3 = s1 * 0x1p-8f;
     const uint32_t e1 = __builtin_bit_cast(uint32_t, s1) >> 23;
     const uint32_t scale = finite ? (e1 | ((e1 - 4u) << 8) | ((e1 - 8u) << 16)) : 0x00FFFFFFu;
+    // residuals pair by pair (v_pk_add_f16): a subtraction of whole 32-element vectors is scalarised by the compiler
+    auto minus = [](const half32_t &a, const half32_t &b) {
+        const v16u_t aw = __builtin_bit_cast(v16u_t, a), bw = __builtin_bit_cast(v16u_t, b);
+        v16u_t rw;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const uint32_t ae = aw[e], be = bw[e];
+            rw[e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, ae) - __builtin_bit_cast(half2_t, be));
+        }
+        return __builtin_bit_cast(half32_t, rw);
+    };
     const v6u_t t1 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(z, s1);
-    const half32_t r1 = z - __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t1, s1);
+    const half32_t r1 = minus(z, __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t1, s1));
     const v6u_t t2 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(r1, s2);
-    const half32_t r2 = r1 - __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t2, s2);
+    const half32_t r2 = minus(r1, __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(t2, s2));
     const v6u_t t3 = __builtin_amdgcn_cvt_scalef32_pk32_fp6_f16(r2, s3);
     const int hq = 4 * h + q, cl = 16 * g + 4 * j + k;             // operand set and consumer lane this thread feeds
     char *op = zbuf + hq * 3 * MX_OPERAND;
@@ -238,7 +251,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     };
     auto produce_write = [&](int buf) {
         if (!l_xlive) px = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
-        mx_produce_finish(zl + buf * MX_ZBUF, stage, pv, px, ph, pj, lane, K);
+        mx_produce_finish(zl + buf * MX_ZBUF, stage, pv, px, ph, pj, lane);
     };
 
     // ---- one (half, position) pass: per row tile four ANDs and three MFMAs ---------------------------
@@ -246,6 +259,12 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // sign position, whose codes need the OR) every word is re-requested for the next unit right
     // behind its last use, so the sign bytes need one register set, not two.  (Unconditionally: a
     // branch around a load makes the compiler keep both values and wait for everything in flight.)
+    // (w & 0x88888888) | 0x22222222 as ONE v_and_or_b32: VOP3 takes no literal and one scalar operand, so the mask is
+    // pinned into a scalar register and the code of 1.0 into a vector register (empty asm statements the optimiser
+    // cannot see through; the merge itself stays an ordinary expression the hazard recogniser can see)
+    uint32_t sign_mask = 0x88888888u, ones_v = 0x22222222u;
+    asm("" : "+s"(sign_mask));
+    asm("" : "+v"(ones_v));
     uint4_t w[R][2];
     uint4_t bk[R];              // T = 2: the sign operands of a position, made for token 0 and used again for token 1
     auto pass = [&](const uint4_t &p0, const uint4_t &p1, const uint4_t &p2, const uint2_t &r0, const uint2_t &r1,
@@ -253,7 +272,6 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
         constexpr int h = decltype(hq_const)::value >> 2, q = decltype(hq_const)::value & 3;
         constexpr int wi = T == 1 ? h : 0, ti = T == 1 ? 0 : h;      // sign word set and token of this pass
         constexpr bool last_use = q == 3 && (T == 1 || h == 1);
-        constexpr uint32_t ONES = 0x22222222u;           // 1.0 in every nibble
         constexpr uint32_t mask = 0x11111111u << q;
         // B scale that makes a set bit worth 2 (q < 3: codes 2, 1, 0.5) or the sign code worth 1
         constexpr uint32_t sb = q == 3 ? 127u : 129u - q;
@@ -266,7 +284,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                     b[jr] = bk[j0 + jr];
                 } else {
 #pragma unroll
-                    for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? ((w[j0 + jr][wi][p] & mask) | ONES) : (w[j0 + jr][wi][p] & mask);
+                    for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? mx_and_or(w[j0 + jr][wi][p], sign_mask, ones_v) : (w[j0 + jr][wi][p] & mask);
                     if (T == 2) bk[j0 + jr] = b[jr];
                 }
                 if (last_use) w[j0 + jr][wi] = *reinterpret_cast<const uint4_t *>(lq + qoff[j0 + jr] + (wi ? l_h1 : 0));
