@@ -33,9 +33,11 @@ SIGNATURES = {
     "bs_decode_kernel": (_I, [_I, _I, _I, _I, _I]),
     "bs_set_decode_kernel": (_I, [_I]),
     "bs_set_dense_kernel": (_I, [_I]),
+    "bs_set_prefill_kernel": (_I, [_I]),
 }
 DECODE_AUTO, DECODE_F16, DECODE_MX = 0, 1, 2
 DENSE_AUTO, DENSE_OWN, DENSE_LIBRARY = 0, 1, 2
+PREFILL_AUTO, PREFILL_REBUILD, PREFILL_WALKED, PREFILL_PANEL = 0, 1, 2, 3
 STATIC_SCRATCH_BYTES = 64 << 20
 
 

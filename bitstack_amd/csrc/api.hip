@@ -40,6 +40,16 @@ static bool dense_wants_library(int M, int N) {
     return g_dense_kernel == BS_DENSE_LIBRARY && M % 8 == 0 && N % 8 == 0;
 }
 
+// Which kernel runs a forward of 49 tokens or more: by shape (0), or pinned for tests and benchmarks.  Per thread.
+static thread_local int g_prefill_kernel = 0;
+int bs_prefill_mode() { return g_prefill_kernel; }
+
+extern "C" int bs_set_prefill_kernel(int mode) {
+    if (mode < 0 || mode > 3) return BS_ERR_SHAPE;
+    g_prefill_kernel = mode;
+    return BS_OK;
+}
+
 extern "C" int bs_set_dense_kernel(int mode) {
     if (mode < 0 || mode > 2) return BS_ERR_SHAPE;
     g_dense_kernel = mode;

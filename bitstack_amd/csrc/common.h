@@ -84,6 +84,14 @@ int bs_strip_partials(int I, int M, int N, int K, int T);
 int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
                           const int *I, const int *M, float *const *part, float *ssq, const half_t *x,
                           int N, int K, int T, hipStream_t s);
+// panel kernel (panel.hip): the same partial sums for up to 128 tokens, sign tiles decoded into LDS and
+// multiplied on the matrix cores at once; bs_panel_partials = column groups (0: the shape is not taken)
+constexpr int BS_PANEL_MAX_T = 128;
+int bs_panel_partials(int I, int M, int N, int K, int T);
+int bs_launch_panel(const uint8_t *packed, const half_t *u, const half_t *vt, int I, int M, float *part, const half_t *x,
+                    int N, int K, int T, hipStream_t s);
+// which kernel runs a forward of 49 tokens or more (bs_set_prefill_kernel, per thread): values of BS_PREFILL_*
+int bs_prefill_mode();
 // decode-step kernels around the linears (decode_step.hip)
 int bs_launch_argmax(const half_t *x, int64_t *out, int B, int V, hipStream_t s);
 int bs_launch_rmsnorm(const half_t *x, const half_t *weight, half_t *y, int T, int H, float eps, hipStream_t s);

@@ -780,7 +780,7 @@ int pass_tokens(int T) { return T <= 4 ? T : (T + 1) / 2; }
 // From this many tokens on the strip kernel (weight patches rebuilt in registers and
 // multiplied at once) is faster than passes of the factor-through kernel, which needs 16
 // rank-MFMAs per token and patch where the strip kernel needs one for 16 tokens.
-constexpr int STRIP_MIN_T = 5, STRIP_MAX_T = 96;       // (49..96 tokens: the walked variant, single matrices only)
+constexpr int STRIP_MIN_T = 5, STRIP_MAX_T = BS_PANEL_MAX_T;       // (49 tokens and more: the walked and panel kernels, single matrices only)
 
 bool strip_group_ok(const int *I, const int *M, int n, int N, int K, int T) {
     for (int j = 0; j < n; j++)

@@ -20,71 +20,14 @@
 // of w (two thirds of the rebuild's bytes) and no second pass that reads it back; the
 // token count only adds one MFMA per patch and 16 tokens, after the last block.
 #include "common.h"
+#include "rebuild_shared.h"
 
 namespace {
 
-constexpr int SF_COLS = 128;    // columns per strip
-constexpr int VSTRIDE = 16;     // halves per column of the vt image: the 16 ranks
-constexpr int VGROUP_PAD = 4;   // extra halves after every 8 columns
-constexpr int VBLOCK = SF_COLS * VSTRIDE + (SF_COLS / 8) * VGROUP_PAD;   // halves per block
 // Extra halves per token row of the x image: rows then start two banks apart, so the 16 tokens a quarter wave reads
 // (8 bytes each, the same columns) fall on 32 different banks.  (With 8, tokens t and t + 8 shared their banks.)
 // Rows are 8-byte aligned only: the image is written and read in pieces of four halves.
 constexpr int XPAD = 4;
-
-// The 16 sign nibbles as four halves each (+1.0 for a set bit, first column in the top bit), at the very start of
-// LDS and 128-byte aligned: a nibble times 8, OR-ed into the table's address, is where its four signs lie.  16
-// entries of 8 bytes take one pair of banks each and equal nibbles read the same address: no bank conflicts.
-constexpr int SIGN_LUT_HALVES = 64;
-typedef const __attribute__((address_space(3))) half4_t *lds_half4_ptr;
-struct SignTable {
-    uint32_t base;       // LDS address of the table
-    int sh_hi, sh_lo;    // the lane's byte of a sign word is byte g: (word >> sh_hi) & 0x78 addresses the signs of its
-                         // first four columns, (word rotated right by sh_lo) & 0x78 those of the other four
-};
-__device__ __forceinline__ SignTable make_sign_table(half_t *lut, int tid, int g) {
-    if (tid < SIGN_LUT_HALVES) lut[tid] = ((tid >> 2) >> (3 - (tid & 3))) & 1 ? (half_t)1.f : (half_t)-1.f;
-    SignTable st;
-    st.base = (uint32_t)reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) half_t *)lut);
-    st.sh_hi = 8 * g + 1;
-    st.sh_lo = (8 * g - 3) & 31;
-    return st;
-}
-
-// Register sets of (u rows, sign words) a wave's requests rotate through: they run NSETS - 1 (row step, strip,
-// block) triples ahead.  The loops below are written out NSETS triples at a time, so that no set is ever copied
-// into another: a copy waits for the load it copies, which would pull every request back to one triple ahead.
-constexpr int NSETS = 3;
-
-// One block of a 16-row x 128-column patch row: acc[s][j] += sign * (u . vt) for the eight 16 x 16 patches.
-// vb: this lane's fragment of the block's vt image.  All eight fragments and all eight sign vectors are
-// requested first, and every product runs one patch ahead of the FMAs that use it: neither the LDS nor the
-// MFMA latency sits in front of them.
-// FIRST: the sums start here (a zero addend; a plain product would not become a mixed-precision instruction).
-template <bool FIRST>
-__device__ __forceinline__ void rebuild_block(const half_t *vb, const half4_t b, const uint4_t sw, const SignTable st,
-                                              float4_t (&acc)[8]) {
-    half4_t a[8], sv[8];
-#pragma unroll
-    for (int s = 0; s < 8; s++)
-        a[s] = *reinterpret_cast<const half4_t *>(vb + (32 * (s >> 1) + 4 * (s & 1)) * VSTRIDE + 4 * (s >> 1) * VGROUP_PAD);
-    auto lookup = [&](int q) {      // the signs of patches 2q and 2q + 1
-        const uint32_t hi = ((sw[q] >> st.sh_hi) & 0x78u) | st.base;
-        const uint32_t lo = (__builtin_amdgcn_alignbit(sw[q], sw[q], st.sh_lo) & 0x78u) | st.base;
-        sv[2 * q] = *reinterpret_cast<lds_half4_ptr>(hi);
-        sv[2 * q + 1] = *reinterpret_cast<lds_half4_ptr>(lo);
-    };
-    lookup(0);
-    float4_t p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[0], b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-    for (int s = 0; s < 8; s++) {
-        const float4_t p = p_next;
-        if (s + 1 < 8) p_next = __builtin_amdgcn_mfma_f32_16x16x16f16(a[s + 1], b, (float4_t){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-        if (s % 2 == 0 && s < 6) lookup(s / 2 + 1);   // the sign vectors of the next two patches, while these two are used
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[s][j] = __builtin_fmaf(p[j], (float)sv[s][j], FIRST ? 0.f : acc[s][j]);
-    }
-}
 
 // TT = token tiles of 16.  A workgroup takes `sg` (1, 2, 4 or 8) neighbouring strips at once:
 // their vt slices are staged together, and per 16-row step the partial y of all of them
@@ -643,16 +586,33 @@ int launch_tt(const StripGroup &grp, int grid, size_t lds, const half_t *x, int 
 
 }  // namespace
 
+// 49 tokens and more: the walked kernel (49..96 tokens, where its plan says it is worth it) or the panel kernel (up to
+// BS_PANEL_MAX_T tokens); bs_set_prefill_kernel can pin either, or switch both off.
+static int wide_partials(int I, int M, int N, int K, int T) {
+    if (T > WIDE_MAX_T) return 0;
+    // the walked kernel: 32-bit row offsets, and an LDS image of one strip that leaves room for two workgroups
+    if ((int64_t)M * (N >> 3) >= ((int64_t)1 << 32) || (int64_t)M * K * 2 >= ((int64_t)1 << 32)) return 0;
+    const WidePlan p = make_wide_plan(I, M, N, T);
+    const bool worth = p.worth || bs_prefill_mode() == BS_PREFILL_WALKED;
+    return (p.lds * 2 <= 160 * 1024 && worth && p.col_groups <= 1024) ? p.col_groups : 0;
+}
+// 1: walked kernel, 2: panel kernel, 0: neither (the weight is rebuilt)
+static int wide_choice(int I, int M, int N, int K, int T) {
+    const int mode = bs_prefill_mode();
+    if (mode == BS_PREFILL_REBUILD) return 0;
+    const bool walked = wide_partials(I, M, N, K, T) > 0, panel = bs_panel_partials(I, M, N, K, T) > 0;
+    if (mode == BS_PREFILL_WALKED) return walked ? 1 : 0;
+    if (mode == BS_PREFILL_PANEL) return panel ? 2 : 0;
+    return walked ? 1 : panel ? 2 : 0;
+}
+
 // Partial sums per output (groups of strips) when this path takes the shape, else 0.
 int bs_strip_partials(int I, int M, int N, int K, int T) {
-    (void)K;
-    if (I < 1 || M < 1 || T < 1 || T > WIDE_MAX_T || N % SF_COLS != 0) return 0;
+    if (I < 1 || M < 1 || T < 1 || T > BS_PANEL_MAX_T || N % SF_COLS != 0) return 0;
     if ((int64_t)M * N >= ((int64_t)1 << 34)) return 0;
     if (T >= WIDE_MIN_T) {
-        // the walked kernel: 32-bit row offsets, and an LDS image of one strip that leaves room for two workgroups
-        if ((int64_t)M * (N >> 3) >= ((int64_t)1 << 32) || (int64_t)M * K * 2 >= ((int64_t)1 << 32)) return 0;
-        const WidePlan p = make_wide_plan(I, M, N, T);
-        return (p.lds * 2 <= 160 * 1024 && p.worth && p.col_groups <= 1024) ? p.col_groups : 0;
+        const int c = wide_choice(I, M, N, K, T);
+        return c == 1 ? wide_partials(I, M, N, K, T) : c == 2 ? bs_panel_partials(I, M, N, K, T) : 0;
     }
     if (strip_lds(I, token_tiles(T), 1) > 160 * 1024) return 0;
     const StripPlan p = make_strip_plan(I, M, N, T);
@@ -666,9 +626,10 @@ int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *con
                           int N, int K, int T, hipStream_t s) {
     if (n < 1 || n > STRIP_MAX_GROUP || !bs_aligned(x, 16)) return BS_ERR_SHAPE;
     if (T >= WIDE_MIN_T) {
-        // one matrix, no sums of squares: the walked kernel serves bs_forward's 49..128-token calls only
+        // one matrix, no sums of squares: these kernels serve bs_forward's calls only
         if (n != 1 || ssq || bs_strip_partials(I[0], M[0], N, K, T) == 0) return BS_ERR_SHAPE;
         if (!bs_aligned(packed[0], 16) || !bs_aligned(vt[0], 16) || !bs_aligned(u[0], 8)) return BS_ERR_SHAPE;
+        if (wide_choice(I[0], M[0], N, K, T) == 2) return bs_launch_panel(packed[0], u[0], vt[0], I[0], M[0], part[0], x, N, K, T, s);
         const WidePlan p = make_wide_plan(I[0], M[0], N, T);
         const WideMat m{packed[0], u[0], vt[0], part[0], I[0], M[0], p.sg, p.n_chunk, p.row_tiles};
         const int grid = p.row_tiles * p.col_groups;

@@ -100,9 +100,12 @@ int64_t bs_workspace_bytes(int I, int M, int N, int K, int T);
  * multiplied by x at once, the weight never stored; N % 128 == 0; when it does
  * not take the shape, T <= 8 is two GEMV passes); 49 <= T <= 96 the same
  * patches with the strips walked by workgroups of 128 rows, where that beats
- * the next path (N % 128 == 0, vt of all blocks of a strip within 40 KB of
- * LDS, workgroups that fill the chip or at most 6 blocks); larger T rebuilds the
- * weight once into `workspace` and runs a dense MFMA GEMM.  Requires
+ * the next paths (N % 128 == 0, vt of all blocks of a strip within 40 KB of
+ * LDS, workgroups that fill the chip or at most 6 blocks); otherwise, up to
+ * 128 tokens and 8 blocks (N % 128 == 0), the panel kernel: 128 x 128 tiles of
+ * the weight decoded into LDS strip by strip and multiplied on the matrix
+ * cores at once, the weight never stored; larger T rebuilds the weight once
+ * into `workspace` and runs a dense MFMA GEMM.  Requires
  * N % 8 == 0.  `workspace` must hold bs_workspace_bytes(...) bytes, 256-byte
  * aligned; its contents on entry do not matter and it may be reused by the
  * next call on the same stream.
@@ -123,7 +126,8 @@ int bs_forward(const uint8_t *packed, const void *u, const void *vt, const void 
  * the 8B and 70B linear shapes up to 36 blocks and of their 5..8-token forwards
  * up to 12 blocks; the strip kernel at several dozen tokens on the largest
  * matrices and every forward that rebuilds a weight of more than 32 Mi elements
- * (more than 96 tokens, or N not a multiple of 128) need more and are refused.
+ * (more than 128 tokens, more than 8 blocks above 96 tokens, or N not a
+ * multiple of 128) need more and are refused.
  * All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (different streams, different host threads) race; calls on one
  * stream are ordered and safe.  Same results as bs_forward, bit for bit, for
@@ -193,6 +197,21 @@ int bs_set_decode_kernel(int mode);
 #define BS_DENSE_OWN     1
 #define BS_DENSE_LIBRARY 2
 int bs_set_dense_kernel(int mode);
+
+/*
+ * Test and benchmark hook: which kernel runs a bs_forward of 49 tokens or more
+ * where several take the shape.  0 = by shape (the default),
+ * BS_PREFILL_REBUILD = always rebuild the weight and run the dense product,
+ * BS_PREFILL_WALKED = the walked strip kernel wherever it takes the shape
+ * (49..96 tokens), BS_PREFILL_PANEL = the panel kernel wherever it takes the
+ * shape (up to 128 tokens, up to 8 blocks, N % 128 == 0).  bs_workspace_bytes
+ * follows the setting.  Per calling thread, like bs_set_decode_kernel.  No
+ * counterpart in the reference.
+ */
+#define BS_PREFILL_REBUILD 1
+#define BS_PREFILL_WALKED  2
+#define BS_PREFILL_PANEL   3
+int bs_set_prefill_kernel(int mode);
 
 /*
  * y[T, M] = x[T, N] @ w[M, N]^T (+ bias) on MFMA, fp32 accumulation: the

@@ -203,11 +203,11 @@ def test_dense_kernel_setting_moves_the_workspace_size_and_rejects_unknown_modes
         assert lib.bs_workspace_bytes(I, M, N, K, 2048) == weight
         assert lib.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
         assert lib.bs_workspace_bytes(I, M, N, K, 2048) == weight + (64 << 20)
-        assert lib.bs_workspace_bytes(I, M, N, K, 100) == weight + (64 << 20)
+        assert lib.bs_workspace_bytes(I, M, N, K, 200) == weight + (64 << 20)
         assert lib.bs_workspace_bytes(I, M + 1, N, K, 2048) == (M + 1) * N * 2       # M % 8 != 0: never the library
         assert lib.bs_workspace_bytes(I, M, N, K, 1) < weight                        # decode shapes do not rebuild
         assert lib.bs_set_dense_kernel(_lib.DENSE_AUTO) == 0                         # never the library by itself
-        assert lib.bs_workspace_bytes(I, M, N, K, 100) == weight
+        assert lib.bs_workspace_bytes(I, M, N, K, 200) == weight
         assert lib.bs_workspace_bytes(I, M, N, K, 2048) == weight
         ragged = N + 8                                                               # no strip kernel takes this width
         assert lib.bs_workspace_bytes(I, M, ragged, K, 48) == M * ragged * 2

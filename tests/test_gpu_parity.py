@@ -347,16 +347,99 @@ def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K):
     assert_close(y, dense, "vs rebuilt weight x dense kernel", 2e-3, 2e-4)
 
 
-def test_walked_strips_are_declined_where_rebuild_and_dense_kernel_are_faster():
+@pytest.fixture
+def prefill_kernel():
+    """Lets a test pin the kernel of a forward of 49 tokens or more; back to the planner's choice afterwards."""
     L = _lib.lib()
-    rebuilt = lambda M, N: M * N * 2                    # (+ the vendor GEMM's scratch where that multiplies it)
-    assert L.bs_workspace_bytes(8, 14336, 4096, 16, 64) >= rebuilt(14336, 4096)     # 448 workgroups for 512 slots
-    assert L.bs_workspace_bytes(3, 14336, 4096, 16, 64) >= rebuilt(14336, 4096)     # ... and few blocks
-    assert L.bs_workspace_bytes(3, 8192, 4096, 16, 64) < rebuilt(8192, 4096)        # 512 workgroups: taken
-    assert L.bs_workspace_bytes(8, 4096, 14336, 16, 64) < rebuilt(4096, 14336)      # 512 workgroups
-    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 97) >= rebuilt(4096, 4096)       # seven token tiles
-    assert L.bs_workspace_bytes(20, 4096, 4096, 16, 64) >= rebuilt(4096, 4096)      # vt of 20 blocks: no room for two workgroups
-    assert L.bs_workspace_bytes(3, 4096, 4000, 16, 64) >= rebuilt(4096, 4000)       # N not a multiple of 128
+    yield lambda mode: _lib.check(L.bs_set_prefill_kernel(mode), "bs_set_prefill_kernel")
+    L.bs_set_prefill_kernel(_lib.PREFILL_AUTO)
+
+
+# up to 128 tokens: sign tiles decoded into LDS and multiplied at once (128 rows x 128 tokens per workgroup): ragged
+# rows and tokens, ranks below 16, 1..8 blocks, one strip per column group and many, runs of strips that start and
+# end inside a quad of strips (the 64 bytes one sign load brings), a column count that leaves the last group short
+PANEL_CASES = [(2, 128, 128, 49, 16), (3, 1000, 1152, 100, 16), (1, 4096, 4096, 128, 16), (8, 4096, 4096, 127, 16),
+               (3, 8192, 4096, 120, 16), (2, 4096, 14336, 128, 16), (5, 333, 640, 97, 5), (8, 1024, 4096, 128, 16),
+               (4, 130, 2432, 113, 12), (6, 2000, 1024, 97, 1), (7, 700, 512, 120, 16), (8, 14336, 384, 64, 16),
+               (7, 256, 4096, 128, 16), (3, 520, 1664, 77, 16)]
+
+
+@pytest.mark.parametrize("I,M,N,T,K", PANEL_CASES)
+def test_forward_panel_kernel_matches_oracle(I, M, N, T, K, prefill_kernel):
+    print(f"forward panel kernel I={I} M={M} N={N} T={T} K={K}", flush=True)
+    L = _lib.lib()
+    prefill_kernel(_lib.PREFILL_PANEL)
+    # the path is taken: the scratch is g x ([T, M] partial sums + T sums of squares) for g column groups, not the weight
+    need = int(L.bs_workspace_bytes(I, M, N, K, T))
+    groups = need // (T * (M + 1) * 4)
+    assert groups >= 1 and need == (groups * T * (M + 1) * 4 + 255) // 256 * 256
+    q, u, vt, x = synthetic_layer(M, N, I, T, k=K, seed=7 * I + T, signed_factors=True)
+    bias = (torch.randn(M, generator=torch.Generator().manual_seed(T)) * 0.05).half() if T % 2 else None
+    exact, l0 = oracle_refs(q, u, vt, x, bias)
+    qd, ud, vd, xd = q.to(dev()), u.to(dev()), vt.to(dev()), x.to(dev())
+    bd = None if bias is None else bias.to(dev())
+    ws = _lib.workspace(xd.device, need)
+    ws[:ws.numel() // 4 * 4].view(torch.float32).fill_(float("nan"))       # an unwritten partial cannot pass by luck
+    y = IU.bitstack_forward_hip(qd, ud, vd, xd, bd)
+    assert torch.equal(IU.bitstack_forward_hip(qd, ud, vd, xd, bd), y)
+    yn = y.cpu().numpy()
+    assert yn.dtype == np.float16 and yn.shape == (T, M) and np.isfinite(yn).all()
+    assert_close(yn, exact, "vs fp64")
+    if I <= 8:
+        assert_close(yn, l0, "vs level-0 order")
+    # the same rounding points as rebuilding the fp16 weight and multiplying: only the order of the fp32 sums differs
+    prefill_kernel(_lib.PREFILL_REBUILD)
+    assert int(L.bs_workspace_bytes(I, M, N, K, T)) >= M * N * 2
+    dense = IU.bitstack_forward_hip(qd, ud, vd, xd, bd).cpu().numpy()
+    assert_close(yn, dense, "vs rebuilt weight x dense kernel", 2e-3, 2e-4)
+
+
+def test_prefill_kernel_hook_selects_and_rejects(prefill_kernel):
+    L = _lib.lib()
+    rebuilt = 4096 * 4096 * 2
+    prefill_kernel(_lib.PREFILL_REBUILD)
+    for T in (49, 64, 128, 256):
+        assert L.bs_workspace_bytes(8, 4096, 4096, 16, T) == rebuilt
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 48) < rebuilt            # the strip kernel below 49 tokens is not affected
+    prefill_kernel(_lib.PREFILL_PANEL)
+    for T in (49, 64, 128):
+        assert L.bs_workspace_bytes(8, 4096, 4096, 16, T) == (8 * T * 4097 * 4 + 255) // 256 * 256   # partial sums of 8 column groups
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 129) == rebuilt          # beyond its token block
+    assert L.bs_workspace_bytes(9, 4096, 4096, 16, 128) == rebuilt          # more blocks than it keeps sign words for
+    assert L.bs_workspace_bytes(8, 4096, 4000, 16, 128) == 4096 * 4000 * 2   # N not a multiple of 128
+    prefill_kernel(_lib.PREFILL_WALKED)
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 64) < rebuilt
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == rebuilt          # the walked kernel stops at 96 tokens
+    assert L.bs_set_prefill_kernel(4) < 0 and L.bs_set_prefill_kernel(-1) < 0
+
+
+def test_planner_picks_walked_strips_then_panel_then_rebuild(prefill_kernel):
+    """49..96 tokens: the walked strip kernel where its plan expects to win, else the panel kernel, else the
+    rebuilt weight; 97..128 tokens: the panel kernel or the rebuilt weight.  Told apart by the scratch each asks for."""
+    L = _lib.lib()
+    rebuilt = lambda M, N: M * N * 2
+
+    def need(mode, I, M, N, T):
+        prefill_kernel(mode)
+        b = int(L.bs_workspace_bytes(I, M, N, 16, T))
+        prefill_kernel(_lib.PREFILL_AUTO)
+        return b
+
+    def picked(I, M, N, T):
+        auto = need(_lib.PREFILL_AUTO, I, M, N, T)
+        names = [n for n, mode in (("walked", _lib.PREFILL_WALKED), ("panel", _lib.PREFILL_PANEL)) if need(mode, I, M, N, T) == auto != rebuilt(M, N)]
+        return names[0] if names else ("rebuild" if auto == rebuilt(M, N) else "?")
+
+    assert picked(3, 8192, 4096, 64) == "walked"          # 512 workgroups: the walked kernel fills the chip
+    assert picked(8, 4096, 14336, 64) == "walked"
+    assert picked(8, 14336, 4096, 64) == "panel"          # 448 workgroups for 512 slots: the walked kernel declines
+    assert picked(3, 14336, 4096, 64) == "panel"
+    assert picked(20, 4096, 4096, 64) == "rebuild"        # vt of 20 blocks: no room for two walked workgroups, too many for the panel
+    assert picked(8, 4096, 4096, 97) == "panel"           # seven token tiles: beyond the walked kernel
+    assert picked(8, 4096, 4096, 128) == "panel"
+    assert picked(9, 4096, 4096, 128) == "rebuild"
+    assert picked(8, 4096, 4096, 129) == "rebuild"
+    assert picked(3, 4096, 4000, 64) == "rebuild"         # N not a multiple of 128
 
 
 @pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)

@@ -77,10 +77,12 @@ def test_workspace_bytes(L):
     assert L.bs_workspace_bytes(8, 4096, 4100, 16, 1) == -2
     assert L.bs_workspace_bytes(8, 4096, 4096, 20, 1) == -3
     # prefill and odd shapes rebuild the fp16 weight (the vendor GEMM and its 64 MiB only in comparator mode)
-    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 512) == 4096 * 4096 * 2
     assert L.bs_set_dense_kernel(_lib.DENSE_LIBRARY) == 0
-    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == 4096 * 4096 * 2 + (64 << 20)
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 512) == 4096 * 4096 * 2 + (64 << 20)
     assert L.bs_set_dense_kernel(_lib.DENSE_AUTO) == 0
+    # 49..128 tokens: partial sums per column group of the walked / panel kernels, not the weight
+    assert L.bs_workspace_bytes(8, 4096, 4096, 16, 128) == (8 * 128 * 4097 * 4 + 255) // 256 * 256
     assert L.bs_workspace_bytes(8, 4096, 4104, 16, 20) == 4096 * 4104 * 2
     assert L.bs_workspace_bytes(2, 64, 72, 16, 1) == ((64 * 72 * 2 + 255) // 256) * 256
     # decode keeps fp32 partial row sums: a multiple of T * M * 4, far below the weight

@@ -120,7 +120,7 @@ def test_static_scratch_forward_under_graph_replay(I, M, N, T):
 def test_static_scratch_forward_refuses_what_does_not_fit():
     dev = torch.device("cuda:0")
     L = _lib.lib()
-    I, M, N, T = 2, 8192, 8192, 128                          # rebuilt weight: 128 MiB of scratch
+    I, M, N, T = 2, 8192, 8192, 200                          # rebuilt weight: 128 MiB of scratch
     assert L.bs_workspace_bytes(I, M, N, 16, T) > _lib.STATIC_SCRATCH_BYTES
     q, u, vt, x = synthetic_layer(M, N, I, T, seed=1, device=dev)
     st, _ = forward_static(q, u, vt, x)
