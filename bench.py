@@ -38,7 +38,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
-PEAK_CLOCK_HZ = 2.4e9         # MI355X peak engine clock
+# Time one SIMD needs per MFMA when it issues nothing else, measured on this part with a loop of independent MFMAs at
+# two waves per SIMD (the shader clock settles near 1.8 GHz under such a load, so cycle counts at the 2.4 GHz peak clock
+# would flatter the kernel): v_mfma_scale_f32_16x16x128_f8f6f4 (fp6 x fp4) 10.8 ns, v_mfma_f32_16x16x32_f16 8.8 ns.
+MFMA_MX_NS = 10.8
+MFMA_F16_NS = 8.8
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 BLOCKS = [1, 2, 4, 8, 16]
 PREFILL_T = [16, 64, 128, 512, 2048]
@@ -352,22 +356,25 @@ def main():
             tp = sum(perp) * 1e-3
             pre[f"T{T}"] = {"useful_tflops": round(useful / tp / 1e12, 1),
                             "frac_of_f16_mfma_peak": round(useful / tp / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+            pre[f"T{T}"]["kernels"] = sorted({_lib.PATH_NAMES[int(lib.bs_forward_path(L.I, L.M, L.N, 16, L.T))] for L in lp})
             if T >= 512:
-                # beside it, timed the same way (the four layers in turn, events around each call):
-                # the same forwards with this library's own dense kernel forced, and the module's level 3 =
-                # this library's rebuild kernel, then torch's F.linear (hipBLASLt) as in the reference's
-                # levels 2-4; never the headline
+                # beside it, timed the same way (the four layers in turn, events around each call): the same
+                # forwards with the vendor GEMM (hipBLASLt) behind the rebuild - a comparator, never the headline
+                # and never what bs_forward picks by itself - and the module's level 3 = this library's rebuild
+                # kernel, then torch's F.linear, as the reference's levels 2-4 are built
                 import torch.nn.functional as F
                 from bitstack_amd.utils.inference_utils import unpack_and_reconstruct_w_hip
-                lib.bs_set_dense_kernel(_lib.DENSE_OWN)
-                _, own = time_sweep(lp, 3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
-                lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
-                pre[f"T{T}"]["own_dense_kernel_useful_tflops"] = round(useful / (sum(own) * 1e-3) / 1e12, 1)
+                lib.bs_set_dense_kernel(_lib.DENSE_LIBRARY)
+                try:
+                    _, ven = time_sweep(lp, 3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
+                finally:
+                    lib.bs_set_dense_kernel(_lib.DENSE_AUTO)
+                pre[f"T{T}"]["vendor_gemm_comparator_useful_tflops"] = round(useful / (sum(ven) * 1e-3) / 1e12, 1)
                 _, lvl3 = time_fns([(lambda L=L: F.linear(L.x, unpack_and_reconstruct_w_hip(L.q, L.u, L.vt))) for L in lp],
                                    3, 1, per_layer_events=True, warm_ms=PREFILL_WARM_MS)
                 pre[f"T{T}"]["level3_rebuild_plus_torch_linear_useful_tflops"] = round(useful / (sum(lvl3) * 1e-3) / 1e12, 1)
                 pre[f"T{T}"]["us_per_layer"] = {"layers": [f"{L.M}x{L.N}" for L in lp], "default": [round(v * 1e3, 1) for v in perp],
-                                                "own_dense_kernel": [round(v * 1e3, 1) for v in own],
+                                                "vendor_gemm_comparator": [round(v * 1e3, 1) for v in ven],
                                                 "level3": [round(v * 1e3, 1) for v in lvl3]}
             detail += [{"M": L.M, "N": L.N, "I": L.I, "T": T, "us": round(ms * 1e3, 2),
                         "useful_tflops": round((2.0 * L.M * L.N * L.T + 32.0 * L.I * L.M * L.N) / (ms * 1e-3) / 1e12, 1)}
@@ -411,7 +418,7 @@ def main():
         print(json.dumps({"sweep_tokens": {"tokens": a.tokens, "us_per_pass": round(sum(per) * 1e3, 1),
                                            "GBps": round(bt / (sum(per) * 1e-3) / 1e9, 1),
                                            "layers": [{"M": L.M, "N": L.N, "I": L.I, "us": round(ms * 1e3, 2),
-                                                       "kernel": int(lib.bs_decode_kernel(L.I, L.M, L.N, 16, L.T))}
+                                                       "kernel": _lib.PATH_NAMES[int(lib.bs_forward_path(L.I, L.M, L.N, 16, L.T))]}
                                                       for L, ms in zip(lt, per)]}}))
         return
     if a.only == "copy":
@@ -455,9 +462,12 @@ def main():
     sweep_gbs = pass_bytes / (ev_total_ms * 1e-3) / 1e9
     def kernel_name(L):
         waves, r, grid, _ = _lib.decode_plan(L.I, L.M, L.N, 16, L.T)
-        if lib.bs_decode_kernel(L.I, L.M, L.N, 16, L.T) == _lib.DECODE_MX:
+        path = int(lib.bs_forward_path(L.I, L.M, L.N, 16, L.T))
+        if path == _lib.PATH_DECODE_MX:
             return "gemv_mx_kernel<R=%d>" % r, grid
-        return "gemv_kernel<T=%d,WAVES=%d,R=%d>" % (L.T, waves, r), grid
+        if path == _lib.PATH_DECODE_F16:
+            return "gemv_kernel<T=%d,WAVES=%d,R=%d>" % (L.T, waves, r), grid
+        return _lib.PATH_NAMES[path], 0
 
     detail = [{"M": L.M, "N": L.N, "I": L.I, "T": L.T, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1),
@@ -475,10 +485,21 @@ def main():
     # measured on one of THIS kernel's launches (profiles/decode_traffic_counters.txt, a "ratio:" line per kernel)
     traffic_ratio, traffic_note = None, "no counter run on record for this kernel"
     try:
+        import hashlib
+        def source_id(name):
+            with open(os.path.join(ROOT, "bitstack_amd", "csrc", name), "rb") as f:
+                return hashlib.sha256(f.read()).hexdigest()[:12]
         with open(os.path.join(ROOT, "profiles", "decode_traffic_counters.txt")) as f:
-            for line in f:
-                parts = line.split()
-                if len(parts) >= 3 and parts[0] == "ratio:" and parts[1] == dom:
+            lines = f.read().splitlines()
+        # "source: <file> <sha256[:12]>" lines say which kernel sources the counters were collected on; a ratio is only
+        # used while those files are unchanged
+        stale = [p[1] for p in (l.split() for l in lines) if len(p) == 3 and p[0] == "source:" and source_id(p[1]) != p[2]]
+        for line in lines:
+            parts = line.split()
+            if len(parts) >= 3 and parts[0] == "ratio:" and parts[1] == dom:
+                if stale:
+                    traffic_note = "the counter run on record was made on another version of " + ", ".join(stale) + ": not used"
+                else:
                     traffic_ratio = float(parts[2])
                     traffic_note = ("HBM bytes per launch = algorithmic x %.2f, the (FETCH_SIZE + WRITE_SIZE) / algorithmic ratio of %s "
                                     "(profiles/decode_traffic_counters.txt)" % (traffic_ratio, " ".join(parts[3:])))
@@ -487,13 +508,12 @@ def main():
     # What bounds it, from this run's own numbers: a least-squares line us = fixed + bytes / rate through the
     # kernel's launches separates the per-launch cost from the streaming rate; the floors are the HBM time of the
     # bytes and the matrix-core issue time of the contraction (16 MACs per sign bit; the block-scaled kernel issues
-    # three 16x16x128 MFMAs of 16 + 4 cycles per 16 x 128 signs, the fp16 kernel four 16x16x32 MFMAs of 16 cycles
-    # per 16 x 128 signs, on 1024 SIMDs at the 2.4 GHz peak clock).
-    clock_hz = PEAK_CLOCK_HZ
+    # three 16x16x128 MFMAs per 16 x 128 signs, the fp16 kernel four 16x16x32 MFMAs, on 1024 SIMDs at the measured
+    # time per MFMA).
     def mfma_floor_us(L):
         tiles = L.I * L.M * L.N / (16.0 * 128.0)
-        cycles = tiles * (60.0 if "mx" in dom else 64.0)
-        return cycles / 1024.0 / clock_hz * 1e6
+        ns = tiles * (3 * MFMA_MX_NS if "mx" in dom else 4 * MFMA_F16_NS)
+        return ns / 1024.0 / 1e3
     xs, ys = [L.bytes for L, _ in dom_runs], [ms * 1e3 for _, ms in dom_runs]
     if len(xs) >= 2 and max(xs) > min(xs):
         mx_, my_ = sum(xs) / len(xs), sum(ys) / len(ys)
@@ -507,6 +527,17 @@ def main():
     shares = {"fixed cost per forward (two launches, pipeline fill and drain)": fixed_us or 0.0,
               "matrix-core issue time of the contraction": mfma_floor, "HBM time of the bytes": hbm_floor}
     limiter = max(shares, key=shares.get)
+    # the roofline this kernel is priced against: the larger of its two machine floors (HBM time of its bytes, matrix-core
+    # issue time of its MFMAs); the fixed cost per forward is overhead under either
+    bound = "mfma" if mfma_floor > hbm_floor else "hbm"
+    if bound == "mfma":
+        # issued matrix-core flops of the contraction (16 MACs per sign bit and term) against the dense peak of the
+        # instruction family the kernel runs on
+        terms = 3.0 if "mx" in dom else 1.0
+        flops = sum(2.0 * 16 * terms * L.I * L.M * L.N for L, _ in dom_runs)
+        roof_achieved, roof_peak, roof_unit = flops / (dom_ms * 1e-3) / 1e12, (10100.0 if "mx" in dom else MFMA_F16_PEAK_TFLOPS), "TFLOP/s"
+    else:
+        roof_achieved, roof_peak, roof_unit = achieved, HBM_PEAK_GBS, "GB/s"
     limiter_note = ("of %.1f us per forward: %.1f us fixed (intercept of the line through this kernel's launches), %.1f us MFMA "
                     "issue floor, %.1f us HBM floor; streaming rate beyond the fixed cost %s GB/s -> largest share: %s"
                     % (avg_us, fixed_us or 0.0, mfma_floor, hbm_floor,
@@ -522,8 +553,10 @@ def main():
                    "layers_per_step": len(layers), "algorithmic_MB_per_step": round(pass_bytes / 1e6, 1),
                    "launch": launch},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "roofline": {"bound": bound, "achieved": round(roof_achieved, 1), "peak": roof_peak, "unit": roof_unit,
+                     "frac": round(roof_achieved / roof_peak, 4),
+                     "frac_of_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),
+                     "frac_of_mfma_issue_floor": round(mfma_floor / avg_us, 4),
                      "traffic": None if traffic_ratio is None else round(dom_bytes / dom_n * traffic_ratio),
                      "kernel": dom + " (+ its gemv_reduce_flat_kernel), the instantiation with the most time in the pass",
                      "launches_per_step": dom_n,
@@ -545,9 +578,12 @@ def main():
         b2 = sum(L.bytes for L in l2)
         t2 = sum(per2) * 1e-3
         lib.bs_set_decode_kernel(_lib.DECODE_F16)
-        _, per2f = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
-        lib.bs_set_decode_kernel(_lib.DECODE_AUTO)
+        try:
+            _, per2f = time_sweep(l2, max(3, a.steps // 2), 1, per_layer_events=True, warm_ms=SIDE_WARM_MS)
+        finally:
+            lib.bs_set_decode_kernel(_lib.DECODE_AUTO)
         out["t2"] = {"GBps": round(b2 / t2 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b2 / t2 / 1e9 / HBM_PEAK_GBS, 2),
+                     "kernels": sorted({kernel_name(L)[0] for L in l2}),
                      "GBps_fp16_kernel_forced": round(b2 / (sum(per2f) * 1e-3) / 1e9, 1)}
         detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 2, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l2, per2)]
@@ -558,7 +594,8 @@ def main():
         b4 = sum(L.bytes for L in l4)
         flops4 = sum(2.0 * 16 * L.I * L.M * L.N * L.T for L in l4)
         t4 = sum(per4) * 1e-3
-        out["t4"] = {"GBps": round(b4 / t4 / 1e9, 1), "mfma_tflops_issued": round(flops4 / t4 / 1e12, 1),
+        out["t4"] = {"GBps": round(b4 / t4 / 1e9, 1), "kernels": sorted({kernel_name(L)[0] for L in l4}),
+                     "mfma_tflops_issued": round(flops4 / t4 / 1e12, 1),
                      "frac_of_f16_mfma_peak": round(flops4 / t4 / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
         detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 4, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l4, per4)]
@@ -569,7 +606,7 @@ def main():
         b16 = sum(L.bytes for L in l16)
         t16 = sum(per16) * 1e-3
         out["t16"] = {"GBps": round(b16 / t16 / 1e9, 1), "pct_of_hbm_peak": round(100.0 * b16 / t16 / 1e9 / HBM_PEAK_GBS, 2),
-                      "kernel": "strip_forward_kernel<1,8> + gemv_reduce_flat_kernel"}
+                      "kernels": sorted({kernel_name(L)[0] for L in l16}) + ["gemv_reduce_flat_kernel"]}
         detail += [{"M": L.M, "N": L.N, "I": L.I, "T": 16, "bytes": L.bytes, "us": round(ms * 1e3, 2),
                     "GBps": round(L.bytes / (ms * 1e-3) / 1e9, 1)} for L, ms in zip(l16, per16)]
         del l16

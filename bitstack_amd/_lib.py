@@ -34,10 +34,14 @@ SIGNATURES = {
     "bs_set_decode_kernel": (_I, [_I]),
     "bs_set_dense_kernel": (_I, [_I]),
     "bs_set_prefill_kernel": (_I, [_I]),
+    "bs_forward_path": (_I, [_I, _I, _I, _I, _I]),
 }
 DECODE_AUTO, DECODE_F16, DECODE_MX = 0, 1, 2
 DENSE_AUTO, DENSE_OWN, DENSE_LIBRARY = 0, 1, 2
 PREFILL_AUTO, PREFILL_REBUILD, PREFILL_WALKED, PREFILL_PANEL = 0, 1, 2, 3
+PATH_NAMES = {0: "rebuild + dense", 1: "gemv_kernel (fp16 MFMA)", 2: "gemv_mx_kernel (fp4 x fp6 MFMA)", 3: "strip_forward_kernel",
+              4: "strip_wide_kernel", 5: "panel_forward_kernel"}
+PATH_REBUILD, PATH_DECODE_F16, PATH_DECODE_MX, PATH_STRIP, PATH_WALKED, PATH_PANEL = range(6)
 STATIC_SCRATCH_BYTES = 64 << 20
 
 

@@ -86,6 +86,13 @@ extern "C" int bs_decode_kernel(int I, int M, int N, int K, int T) {
 
 extern "C" int bs_set_decode_kernel(int mode) { return bs_gemv_set_kernel(mode); }
 
+extern "C" int bs_forward_path(int I, int M, int N, int K, int T) {
+    int st = forward_dims(I, M, N, K, T);
+    if (st != BS_OK) return st;
+    if (T == 0 || I == 0) return BS_PATH_REBUILD;      // (no blocks: the weight is zero; the forward still goes through the dense path)
+    return bs_gemv_forward_path(I, M, N, K, T);
+}
+
 static int forward_impl(const uint8_t *packed, const void *u, const void *vt, const void *x,
                         const void *bias, void *y, int I, int M, int N, int K, int T,
                         void *workspace, int64_t workspace_bytes, void *stream, bool library_ok) {

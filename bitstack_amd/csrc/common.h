@@ -71,6 +71,7 @@ int bs_launch_gemv(const uint8_t *packed, const half_t *u, const half_t *vt, con
 int64_t bs_gemv_workspace_bytes(int I, int M, int N, int K, int T);
 void bs_gemv_plan_info(int I, int M, int N, int K, int T, int *waves, int *row_tiles_per_wave, int *grid, int *kmax);
 int bs_gemv_plan_kernel(int I, int M, int N, int K, int T);
+int bs_gemv_forward_path(int I, int M, int N, int K, int T);
 int bs_gemv_set_kernel(int mode);
 // epilogues of the grouped decode forward (values of BS_EPI_* in the public header)
 enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
@@ -81,6 +82,7 @@ int bs_launch_gemv_group(int n, const uint8_t *const *packed, const half_t *cons
                          int64_t workspace_bytes, hipStream_t s);
 // strip kernel (strip.hip): partial sums part[strip, t, m] of x . w^T with w rebuilt in registers
 int bs_strip_partials(int I, int M, int N, int K, int T);
+int bs_strip_kernel_choice(int I, int M, int N, int K, int T);
 int bs_launch_strip_group(int n, const uint8_t *const *packed, const half_t *const *u, const half_t *const *vt,
                           const int *I, const int *M, float *const *part, float *ssq, const half_t *x,
                           int N, int K, int T, hipStream_t s);

@@ -969,6 +969,17 @@ void bs_gemv_plan_info(int I, int M, int N, int K, int T, int *waves, int *row_t
     *kmax = p.kmax[0];
 }
 
+// The kernel family a single-matrix forward of these dimensions runs on (values of BS_PATH_* in the public header).
+int bs_gemv_forward_path(int I, int M, int N, int K, int T) {
+    const int path = group_path(&I, &M, 1, N, K, T);
+    if (path < 0) return BS_PATH_REBUILD;
+    if (path == 1) {
+        const int c = bs_strip_kernel_choice(I, M, N, K, T);
+        return c == 1 ? BS_PATH_STRIP : c == 2 ? BS_PATH_WALKED : BS_PATH_PANEL;
+    }
+    return make_plan(&I, &M, 1, N, K, pass_tokens(T)).mx ? BS_PATH_DECODE_MX : BS_PATH_DECODE_F16;
+}
+
 // 0: not a decode-kernel shape, 1: gemv_kernel (fp16 MFMA), 2: gemv_mx_kernel (block-scaled fp4 x fp6 MFMA)
 int bs_gemv_plan_kernel(int I, int M, int N, int K, int T) {
     if (group_path(&I, &M, 1, N, K, T) != 0) return 0;

@@ -606,6 +606,14 @@ static int wide_choice(int I, int M, int N, int K, int T) {
     return walked ? 1 : panel ? 2 : 0;
 }
 
+// Which of this family's kernels a forward of these dimensions runs: 0 none, 1 strip_forward_kernel (5..48 tokens),
+// 2 strip_wide_kernel (the walked strips), 3 the panel kernel.
+int bs_strip_kernel_choice(int I, int M, int N, int K, int T) {
+    if (bs_strip_partials(I, M, N, K, T) == 0) return 0;
+    if (T < WIDE_MIN_T) return 1;
+    return wide_choice(I, M, N, K, T) == 1 ? 2 : 3;
+}
+
 // Partial sums per output (groups of strips) when this path takes the shape, else 0.
 int bs_strip_partials(int I, int M, int N, int K, int T) {
     if (I < 1 || M < 1 || T < 1 || T > BS_PANEL_MAX_T || N % SF_COLS != 0) return 0;

@@ -168,6 +168,21 @@ int bs_decode_plan(int I, int M, int N, int K, int T, int *waves, int *row_tiles
 int bs_decode_kernel(int I, int M, int N, int K, int T);
 
 /*
+ * Introspection for benchmarks and tests: the kernel family bs_forward runs for
+ * these dimensions under the calling thread's hook settings (for 5..8 tokens
+ * on the decode kernels: that of the first pass).  Negative = error status.
+ * No counterpart in the reference (its fused_level is chosen by the caller,
+ * bitstack/modules/BitStackLinear.py:116-157).
+ */
+#define BS_PATH_REBUILD    0   /* weight rebuilt into the workspace, then the dense product */
+#define BS_PATH_DECODE_F16 1   /* gemv_kernel: packed-sign GEMV on fp16 MFMA, 1..4 tokens per pass */
+#define BS_PATH_DECODE_MX  2   /* gemv_mx_kernel: the same on the block-scaled fp4 x fp6 MFMA, 1..2 tokens */
+#define BS_PATH_STRIP      3   /* strip_forward_kernel: 5..48 tokens, patches rebuilt in registers */
+#define BS_PATH_WALKED     4   /* strip_wide_kernel: 49..96 tokens, strips walked by 128-row workgroups */
+#define BS_PATH_PANEL      5   /* panel_forward_kernel: up to 128 tokens, W tiles decoded into LDS */
+int bs_forward_path(int I, int M, int N, int K, int T);
+
+/*
  * Test and benchmark hook: 0 = choose the decode kernel of one- and two-token
  * passes by shape (the default), BS_DECODE_F16 = always the fp16 kernel,
  * BS_DECODE_MX = the block-scaled kernel wherever it takes the shape

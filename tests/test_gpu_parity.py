@@ -415,31 +415,28 @@ def test_prefill_kernel_hook_selects_and_rejects(prefill_kernel):
 
 def test_planner_picks_walked_strips_then_panel_then_rebuild(prefill_kernel):
     """49..96 tokens: the walked strip kernel where its plan expects to win, else the panel kernel, else the
-    rebuilt weight; 97..128 tokens: the panel kernel or the rebuilt weight.  Told apart by the scratch each asks for."""
+    rebuilt weight; 97..128 tokens: the panel kernel or the rebuilt weight; the hook pins each."""
     L = _lib.lib()
-    rebuilt = lambda M, N: M * N * 2
-
-    def need(mode, I, M, N, T):
-        prefill_kernel(mode)
-        b = int(L.bs_workspace_bytes(I, M, N, 16, T))
-        prefill_kernel(_lib.PREFILL_AUTO)
-        return b
-
-    def picked(I, M, N, T):
-        auto = need(_lib.PREFILL_AUTO, I, M, N, T)
-        names = [n for n, mode in (("walked", _lib.PREFILL_WALKED), ("panel", _lib.PREFILL_PANEL)) if need(mode, I, M, N, T) == auto != rebuilt(M, N)]
-        return names[0] if names else ("rebuild" if auto == rebuilt(M, N) else "?")
-
-    assert picked(3, 8192, 4096, 64) == "walked"          # 512 workgroups: the walked kernel fills the chip
-    assert picked(8, 4096, 14336, 64) == "walked"
-    assert picked(8, 14336, 4096, 64) == "panel"          # 448 workgroups for 512 slots: the walked kernel declines
-    assert picked(3, 14336, 4096, 64) == "panel"
-    assert picked(20, 4096, 4096, 64) == "rebuild"        # vt of 20 blocks: no room for two walked workgroups, too many for the panel
-    assert picked(8, 4096, 4096, 97) == "panel"           # seven token tiles: beyond the walked kernel
-    assert picked(8, 4096, 4096, 128) == "panel"
-    assert picked(9, 4096, 4096, 128) == "rebuild"
-    assert picked(8, 4096, 4096, 129) == "rebuild"
-    assert picked(3, 4096, 4000, 64) == "rebuild"         # N not a multiple of 128
+    path = lambda I, M, N, T: L.bs_forward_path(I, M, N, 16, T)
+    assert path(3, 8192, 4096, 64) == _lib.PATH_WALKED        # 512 workgroups: the walked kernel fills the chip
+    assert path(8, 4096, 14336, 64) == _lib.PATH_WALKED
+    assert path(8, 14336, 4096, 64) == _lib.PATH_PANEL        # 448 workgroups for 512 slots: the walked kernel declines
+    assert path(3, 14336, 4096, 64) == _lib.PATH_PANEL
+    assert path(20, 4096, 4096, 64) == _lib.PATH_REBUILD      # vt of 20 blocks: no room for two walked workgroups, too many for the panel
+    assert path(8, 4096, 4096, 97) == _lib.PATH_PANEL         # seven token tiles: beyond the walked kernel
+    assert path(8, 4096, 4096, 128) == _lib.PATH_PANEL
+    assert path(9, 4096, 4096, 128) == _lib.PATH_REBUILD
+    assert path(8, 4096, 4096, 129) == _lib.PATH_REBUILD
+    assert path(3, 4096, 4000, 64) == _lib.PATH_REBUILD       # N not a multiple of 128
+    assert path(2, 4096, 4096, 1) == _lib.PATH_DECODE_F16 and path(16, 4096, 4096, 1) == _lib.PATH_DECODE_MX
+    assert path(4, 4096, 4096, 16) == _lib.PATH_STRIP and path(4, 4096, 4104, 16) == _lib.PATH_REBUILD
+    prefill_kernel(_lib.PREFILL_REBUILD)
+    assert path(8, 4096, 4096, 64) == _lib.PATH_REBUILD and path(4, 4096, 4096, 16) == _lib.PATH_STRIP
+    prefill_kernel(_lib.PREFILL_PANEL)
+    assert path(8, 4096, 4096, 64) == _lib.PATH_PANEL
+    prefill_kernel(_lib.PREFILL_WALKED)
+    assert path(8, 14336, 4096, 64) == _lib.PATH_WALKED       # pinned where its own plan would decline
+    assert path(8, 4096, 4096, 128) == _lib.PATH_REBUILD
 
 
 @pytest.mark.parametrize("I,M,N,T,K", STRIP_CASES)
