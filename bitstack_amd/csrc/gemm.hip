@@ -8,14 +8,16 @@
 // More than 128 tokens: linear_f16_kernel, WT x WF waves of AT x AF MFMA tiles each,
 // k-steps of GK columns through two LDS buffers; rows are padded by 8 halves so that
 // the lanes served per LDS cycle hit disjoint banks.  Four shapes are instantiated:
-// 256 x 256 (8 waves of 128 x 64, GK = 32) and 128 x 256 (8 waves of 64 x 64) for
+// 256 x 256 (8 waves of 128 x 64; GK = 64 with two register sets of pieces in flight when N % 64 == 0 - a row's 128
+// bytes of a k-step are one cache line, fetched once; GK = 32 took every line from L2 twice, the halves a step apart and
+// the L1 too small to keep them - else GK = 32 with three sets) and 128 x 256 (8 waves of 64 x 64) for
 // grids that cover the chip, 128 x 128 and 64 x 64 (4 waves, two workgroups per CU,
 // the latter with GK = 128: half as many barriers) for the smaller ones; the launcher
 // takes the largest tile whose grid still has about 160 workgroups.
 // The loop is software-pipelined at three levels, all through registers:
-//   - global requests run three k-steps ahead through three register sets, all of
-//     them unconditional with a scalar base and a 32-bit lane offset;
-//   - the LDS writes of step s + 1 and the requests of step s + 3 are cut into one
+//   - global requests run NS (three, or two) k-steps ahead through NS register sets, all
+//     of them unconditional with a scalar base and a 32-bit lane offset;
+//   - the LDS writes of step s + 1 and the requests of step s + NS are cut into one
 //     portion per MFMA group instead of one burst per step;
 //   - MFMA fragments are read from LDS one group ahead of use, the first group of the
 //     next step right behind the barrier.
@@ -52,7 +54,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 __host__ __device__ constexpr bool lds_swizzled(int gk) { return gk == 32; }
 __host__ __device__ constexpr int lds_stride(int gk) { return lds_swizzled(gk) ? gk : gk + 8; }
 
-template <int WT, int WF, int AT, int AF, int GK, bool KTAIL>
+template <int WT, int WF, int AT, int AF, int GK, bool KTAIL, int NS = 3>
 __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     const half_t *__restrict__ x, const half_t *__restrict__ w, const half_t *__restrict__ bias,
     half_t *__restrict__ y, int T, int M, int N) {
@@ -81,6 +83,10 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
     const char *xt = reinterpret_cast<const char *>(x + (int64_t)t0 * N);
     const char *wt_ = reinterpret_cast<const char *>(w + (int64_t)m0 * N);
     const int lrow = tid / PPR, lpiece = tid % PPR;
+    // raw buffer descriptors over the two tile origins (no stride, no range limit short of 4 GiB: offsets are checked
+    // by construction - rows are clamped to the tile, k-steps to the contracted range)
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void *)xt, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void *)wt_, 0, -1, 0x00020000);
     uint32_t off[PER_THREAD];
     int dst[PER_THREAD];
 #pragma unroll
@@ -101,13 +107,13 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
             for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
 
     const int steps = (N + GK - 1) / GK;
-    // Two register sets: while step s is multiplied, the pieces of step s + 1 are already
-    // in one set (in flight or landed) and those of step s + 2 are requested into the other.
+    // NS register sets: while step s is multiplied, the pieces of step s + 1 are in one set
+    // (landed, on their way to LDS) and those of the steps up to s + NS in flight into the others.
     // Every request is unconditional (past the end the last step is requested again), so
     // the compiler's count of outstanding loads is exact and a wait for one set never
     // drains the other.  KTAIL (N not a multiple of GK): pieces beyond column N are read
     // from column 0 instead and replaced by zeros.
-    uint4_t stage[3][PER_THREAD];
+    uint4_t stage[NS][PER_THREAD];
     // part `part` of `parts` of the pieces of one step (the whole step: 0 of 1)
     auto fetch = [&](auto setc, int step_, auto partc, auto partsc) {
         constexpr int set = decltype(setc)::value, part = decltype(partc)::value, parts = decltype(partsc)::value;
@@ -122,10 +128,12 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
                 stage[set][j] = in ? v : (uint4_t){0, 0, 0, 0};
             }
         } else {
-            const char *xs = xt + (int64_t)step * (GK * 2), *ws = wt_ + (int64_t)step * (GK * 2);
+            // buffer loads: descriptor (tile origin) + 32-bit lane offset + scalar k offset - no 64-bit address arithmetic
+            // per request (4-7 % of the kernel's time with flat global loads)
+            const int koff = step * (GK * 2);
 #pragma unroll
             for (int j = j0; j < j1; j++)
-                stage[set][j] = *reinterpret_cast<const uint4_t *>((j < JX ? xs : ws) + off[j]);
+                stage[set][j] = __builtin_amdgcn_raw_buffer_load_b128(j < JX ? rx : rw, (int)off[j], koff, 0);
         }
     };
     // part `part` of `parts` of a register set goes to LDS (the whole set: 0 of 1)
@@ -179,14 +187,14 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
         constexpr int buf = decltype(bufc)::value;
         static_for<NK / 2>([&](auto hc) {
             constexpr int kk = 2 * decltype(hc)::value;
-            fetch(cur, step + 3, std::integral_constant<int, kk>{}, PF{});   // set `cur` was emptied into LDS a step ago
+            fetch(cur, step + NS, std::integral_constant<int, kk>{}, PF{});   // set `cur` was emptied into LDS a step ago
             load_frags(S1{}, buf, kk + 1);
             stash(nxt, buf ^ 1, std::integral_constant<int, kk>{}, PS{});    // after the last step: a copy nobody reads
             __builtin_amdgcn_sched_barrier(0);
             mfmas(S0{});
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (kk + 2 < NK) {
-                fetch(cur, step + 3, std::integral_constant<int, kk + 1>{}, PF{});
+                fetch(cur, step + NS, std::integral_constant<int, kk + 1>{}, PF{});
                 load_frags(S0{}, buf, kk + 2);
                 stash(nxt, buf ^ 1, std::integral_constant<int, kk + 1>{}, PS{});
                 __builtin_amdgcn_sched_barrier(0);
@@ -195,7 +203,7 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
             }
         });
         __syncthreads();
-        fetch(cur, step + 3, std::integral_constant<int, NK - 1>{}, PF{});
+        fetch(cur, step + NS, std::integral_constant<int, NK - 1>{}, PF{});
         load_frags(S0{}, buf ^ 1, 0);
         __builtin_amdgcn_sched_barrier(0);
         mfmas(S1{});
@@ -204,17 +212,24 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
 
     fetch(S0{}, 0, S0{}, S1{});
     fetch(S1{}, 1, S0{}, S1{});
-    fetch(S2{}, 2, S0{}, S1{});
+    if constexpr (NS == 3) fetch(S2{}, 2, S0{}, S1{});
     stash(S0{}, 0, S0{}, S1{});
     __syncthreads();
     load_frags(S0{}, 0, 0);
-    for (int step = 0; step < steps; step += 6) {
-        one_step(S0{}, S1{}, S0{}, step);
-        if (step + 1 < steps) one_step(S1{}, S2{}, S1{}, step + 1);
-        if (step + 2 < steps) one_step(S2{}, S0{}, S0{}, step + 2);
-        if (step + 3 < steps) one_step(S0{}, S1{}, S1{}, step + 3);
-        if (step + 4 < steps) one_step(S1{}, S2{}, S0{}, step + 4);
-        if (step + 5 < steps) one_step(S2{}, S0{}, S1{}, step + 5);
+    if constexpr (NS == 3) {
+        for (int step = 0; step < steps; step += 6) {
+            one_step(S0{}, S1{}, S0{}, step);
+            if (step + 1 < steps) one_step(S1{}, S2{}, S1{}, step + 1);
+            if (step + 2 < steps) one_step(S2{}, S0{}, S0{}, step + 2);
+            if (step + 3 < steps) one_step(S0{}, S1{}, S1{}, step + 3);
+            if (step + 4 < steps) one_step(S1{}, S2{}, S0{}, step + 4);
+            if (step + 5 < steps) one_step(S2{}, S0{}, S1{}, step + 5);
+        }
+    } else {
+        for (int step = 0; step < steps; step += 2) {
+            one_step(S0{}, S1{}, S0{}, step);
+            if (step + 1 < steps) one_step(S1{}, S0{}, S1{}, step + 1);
+        }
     }
 
     // D[token, feature]: lane holds feature l32, tokens 8 * (v / 4) + 4 * kh + v % 4
@@ -317,20 +332,28 @@ __global__ __launch_bounds__(256) void linear_generic_kernel(
     }
 }
 
-template <int WT, int WF, int AT, int AF, int GK>
+// NS: register sets of pieces in flight.  TAILS: also instantiate the kernel for a contracted range that ends in a partial
+// k-step (false: the caller only comes with N % GK == 0).
+template <int WT, int WF, int AT, int AF, int GK, int NS = 3, bool TAILS = true>
 int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y, int T, int M, int N,
                  hipStream_t s) {
     constexpr int BT = WT * AT * 32, BF = WF * AF * 32;
     constexpr size_t lds = (size_t)2 * (BT + BF) * lds_stride(GK) * sizeof(half_t);
     static bs_lds_grant granted[2][BS_MAX_DEVICES];
-    int st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false>, lds, granted[0]);
-    if (st == BS_OK) st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true>, lds, granted[1]);
+    int st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, false, NS>, lds, granted[0]);
+    if constexpr (TAILS) {
+        if (st == BS_OK) st = bs_allow_lds((const void *)linear_f16_kernel<WT, WF, AT, AF, GK, true, NS>, lds, granted[1]);
+    }
     if (st != BS_OK) return st;
     dim3 grid((unsigned)bs_cdiv(M, BF), (unsigned)bs_cdiv(T, BT));
-    if (N % GK == 0)
-        linear_f16_kernel<WT, WF, AT, AF, GK, false><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
-    else
-        linear_f16_kernel<WT, WF, AT, AF, GK, true><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
+    if (N % GK == 0) {
+        linear_f16_kernel<WT, WF, AT, AF, GK, false, NS><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
+    } else {
+        if constexpr (TAILS)
+            linear_f16_kernel<WT, WF, AT, AF, GK, true, NS><<<grid, 64 * WT * WF, lds, s>>>(x, w, bias, y, T, M, N);
+        else
+            return BS_ERR_SHAPE;
+    }
     return BS_OK;
 }
 
@@ -341,14 +364,14 @@ int launch_tiled(const half_t *x, const half_t *w, const half_t *bias, half_t *y
 // partial k-step.
 struct LinearTile { int bt, bf, gk; };
 static LinearTile linear_tile(int T, int M, int N, bool aligned) {
-    if (!(N % 8 == 0 && aligned)) return {0, 0, 0};
+    if (!(N % 8 == 0 && aligned) || N >= (1 << 23)) return {0, 0, 0};     // (a tile's rows stay within 32-bit byte offsets)
     if (T <= 32 && N % 16 == 0) return {32, 32, 0};                       // linear_skinny_kernel
     if (T <= 128) return M >= 8192 ? LinearTile{128, 64, 64} : LinearTile{128, 32, 128};
     // The largest tile whose grid still covers most of the 256 CUs: 256 x 256 and
     // 128 x 256 (8 waves) move the fewest bytes per flop; 128 x 128 and 64 x 64
     // (4 waves, two workgroups per CU) keep a small problem spread over the chip.
     const auto wgs = [&](int bt, int bf) { return bs_cdiv(T, bt) * bs_cdiv(M, bf); };
-    return wgs(256, 256) >= 160 ? LinearTile{256, 256, 32} :
+    return wgs(256, 256) >= 160 ? LinearTile{256, 256, N % 64 == 0 ? 64 : 32} :
            wgs(128, 256) >= 160 ? LinearTile{128, 256, 64} :
            wgs(128, 128) >= 192 ? LinearTile{128, 128, 64} : LinearTile{64, 64, 128};
 }
@@ -367,6 +390,8 @@ int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, h
         st = launch_tiled<2, 2, 2, 1, 64>(x, w, bias, y, T, M, N, s);
     } else if (tile.bt == 128 && tile.bf == 32) {
         st = launch_tiled<4, 1, 1, 1, 128>(x, w, bias, y, T, M, N, s);
+    } else if (tile.bt == 256 && tile.gk == 64) {
+        st = launch_tiled<2, 4, 4, 2, 64, 2, false>(x, w, bias, y, T, M, N, s);
     } else if (tile.bt == 256) {
         st = launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s);
     } else if (tile.bf == 256) {

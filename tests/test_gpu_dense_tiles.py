@@ -47,6 +47,7 @@ TILE_CASES = [
     (2048, 14336, 4096, (256, 256), 0),
     (2047, 14335, 4096, (256, 256), 0),        # ragged tokens and features
     (1024, 14336, 4104, (256, 256), 1),        # N % 32 != 0
+    (1024, 14336, 4128, (256, 256), 0),        # N % 64 != 0: k-steps of 32
     (16384, 8192, 8192, (256, 256), 0),        # the 70B prefill of 2048 tokens x 8 sequences
     (2048, 4096, 4096, (128, 256), 0),
     (512, 14336, 4096, (128, 256), 0),
