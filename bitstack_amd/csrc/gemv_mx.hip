@@ -62,6 +62,12 @@ constexpr int MX_OPERAND = 64 * 16 + 64 * 8;        // bytes of one (half, q, te
 constexpr int MX_SCALES = 8 * 3 * MX_OPERAND;       // the scale words of a Z buffer follow its 24 operands
 constexpr int MX_ZBUF = MX_SCALES + 8 * 64 * 4;     // bytes per Z buffer
 
+// raw buffer descriptor from a pointer: no stride, no range limit short of 4 GiB (every offset used with it is checked
+// by construction: rows clamped to M, columns to the unit)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t mx_rsrc(const void *p) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, -1, 0x00020000);
+}
+
 __device__ __forceinline__ uint32_t mx_and_or(uint32_t w, uint32_t mask, uint32_t base) { return (w & mask) | base; }
 
 __device__ __forceinline__ float4_t mx_mfma(const uint4_t &a03, const uint2_t &a45, const uint4_t &b, float4_t c,
@@ -211,8 +217,11 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     // Sign words and vt pieces are requested for the unit AFTER the one being multiplied; `qoff`,
     // `lq`, `lv` always describe that unit.
     uint32_t qoff[R];           // this lane's row in each row tile of the wave, as a byte offset within a block
-    const uint8_t *lq;          // packed signs of the block, at the unit's first column
-    const half_t *lv;           // vt of the block: rank 4 pj, this lane's 8 columns of half ph of the unit
+    // Requests are raw buffer loads: a descriptor over the unit's origin (scalar registers), a 32-bit lane offset and a
+    // scalar offset - no 64-bit address arithmetic in the vector unit, which this kernel cannot hide under its MFMAs.
+    __amdgpu_buffer_rsrc_t lq;  // packed signs of the block, from the unit's first column
+    __amdgpu_buffer_rsrc_t lv;  // vt of the block: rank 0, from the first column of half ph of the unit
+    __amdgpu_buffer_rsrc_t lx;  // x (of token ph when T = 2) from the same column
     int l_h1;                   // byte offset of the unit's second half of a row (0 when it lies beyond N)
     bool l_xlive;               // the producer half of this wave lies within N
     auto set_unit = [&](int rowid, int c, bool new_row) {
@@ -225,9 +234,10 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                 qoff[jr] = row * (uint32_t)row_bytes + 16u * g;
             }
         }
-        lq = packed + (int64_t)i * M * row_bytes + c * (UC >> 3);
+        lq = mx_rsrc(packed + (int64_t)i * M * row_bytes + c * (UC >> 3));
         l_h1 = half_cols(c, 1) >> 3;
-        lv = vt + ((int64_t)i * K + 4 * pj) * N + c * UC + half_cols(c, ph) + 8 * lane;    // (4 pj may exceed K - 1: see produce_issue)
+        lv = mx_rsrc(vt + (int64_t)i * K * N + c * UC + half_cols(c, ph));
+        lx = mx_rsrc(x + (T == 2 ? (int64_t)ph * N : 0) + c * UC + half_cols(c, ph));
         l_xlive = T == 2 || c * UC + 512 * ph < N;
     };
 
@@ -246,8 +256,9 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     auto produce_issue = [&](int c) {
         // (ranks beyond K repeat rank K - 1 and are zeroed when the operands are formed: no branch around a load)
 #pragma unroll
-        for (int k = 0; k < 4; k++) pv[k] = *reinterpret_cast<const half8_t *>(lv + (int64_t)(min(4 * pj + k, K - 1) - 4 * pj) * N);
-        px = *reinterpret_cast<const half8_t *>(x + (T == 2 ? (int64_t)ph * N : 0) + c * UC + half_cols(c, ph) + 8 * lane);
+        for (int k = 0; k < 4; k++)
+            pv[k] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(lv, 16 * lane, min(4 * pj + k, K - 1) * N * 2, 0));
+        px = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(lx, 16 * lane, 0, 0));
     };
     auto produce_write = [&](int buf) {
         if (!l_xlive) px = (half8_t){0, 0, 0, 0, 0, 0, 0, 0};
@@ -287,7 +298,7 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
                     for (int p = 0; p < 4; p++) b[jr][p] = q == 3 ? mx_and_or(w[j0 + jr][wi][p], sign_mask, ones_v) : (w[j0 + jr][wi][p] & mask);
                     if (T == 2) bk[j0 + jr] = b[jr];
                 }
-                if (last_use) w[j0 + jr][wi] = *reinterpret_cast<const uint4_t *>(lq + qoff[j0 + jr] + (wi ? l_h1 : 0));
+                if (last_use) w[j0 + jr][wi] = __builtin_amdgcn_raw_buffer_load_b128(lq, (int)qoff[j0 + jr], wi ? l_h1 : 0, 0);
             }
             // term by term over the row tiles: consecutive MFMAs never share an accumulator
 #pragma unroll
@@ -427,10 +438,10 @@ __global__ __launch_bounds__(64 * MX_WAVES, 1) void gemv_mx_kernel(
     produce_issue(c);
     // first halves first: the first four passes need nothing else (requests complete in order)
 #pragma unroll
-    for (int jr = 0; jr < R; jr++) w[jr][0] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr]);
+    for (int jr = 0; jr < R; jr++) w[jr][0] = __builtin_amdgcn_raw_buffer_load_b128(lq, (int)qoff[jr], 0, 0);
     if (T == 1) {
 #pragma unroll
-        for (int jr = 0; jr < R; jr++) w[jr][1] = *reinterpret_cast<const uint4_t *>(lq + qoff[jr] + l_h1);
+        for (int jr = 0; jr < R; jr++) w[jr][1] = __builtin_amdgcn_raw_buffer_load_b128(lq, (int)qoff[jr], l_h1, 0);
     }
     produce_write(0);
     __syncthreads();
