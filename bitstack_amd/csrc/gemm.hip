@@ -15,8 +15,10 @@
 // the latter with GK = 128: half as many barriers) for the smaller ones; the launcher
 // takes the largest tile whose grid still has about 160 workgroups.
 // The loop is software-pipelined at three levels, all through registers:
-//   - global requests run NS (three, or two) k-steps ahead through NS register sets, all
-//     of them unconditional with a scalar base and a 32-bit lane offset;
+//   - global requests run NS k-steps ahead through NS register sets (four where the registers allow it: the
+//     kernel waits for requests more than for anything else, and a fourth set is worth 3 to 13 %; five and six were
+//     no better; two for the 256 x 256 tile in k-steps of 64), all of them unconditional buffer loads: descriptor,
+//     32-bit lane offset, scalar k offset;
 //   - the LDS writes of step s + 1 and the requests of step s + NS are cut into one
 //     portion per MFMA group instead of one burst per step;
 //   - MFMA fragments are read from LDS one group ahead of use, the first group of the
@@ -210,26 +212,20 @@ __global__ __launch_bounds__(64 * WT * WF) void linear_f16_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    fetch(S0{}, 0, S0{}, S1{});
-    fetch(S1{}, 1, S0{}, S1{});
-    if constexpr (NS == 3) fetch(S2{}, 2, S0{}, S1{});
+    // step s: its pieces travel through register set s % NS and are multiplied out of LDS buffer s % 2; the loop is
+    // written out over one period of both, so that every set and buffer index is a constant
+    static_for<NS>([&](auto kc) { fetch(kc, decltype(kc)::value, S0{}, S1{}); });
     stash(S0{}, 0, S0{}, S1{});
     __syncthreads();
     load_frags(S0{}, 0, 0);
-    if constexpr (NS == 3) {
-        for (int step = 0; step < steps; step += 6) {
-            one_step(S0{}, S1{}, S0{}, step);
-            if (step + 1 < steps) one_step(S1{}, S2{}, S1{}, step + 1);
-            if (step + 2 < steps) one_step(S2{}, S0{}, S0{}, step + 2);
-            if (step + 3 < steps) one_step(S0{}, S1{}, S1{}, step + 3);
-            if (step + 4 < steps) one_step(S1{}, S2{}, S0{}, step + 4);
-            if (step + 5 < steps) one_step(S2{}, S0{}, S1{}, step + 5);
-        }
-    } else {
-        for (int step = 0; step < steps; step += 2) {
-            one_step(S0{}, S1{}, S0{}, step);
-            if (step + 1 < steps) one_step(S1{}, S0{}, S1{}, step + 1);
-        }
+    constexpr int PERIOD = NS % 2 == 0 ? NS : 2 * NS;
+    for (int step = 0; step < steps; step += PERIOD) {
+        static_for<PERIOD>([&](auto kc) {
+            constexpr int k = decltype(kc)::value;
+            if (k == 0 || step + k < steps)
+                one_step(std::integral_constant<int, k % NS>{}, std::integral_constant<int, (k + 1) % NS>{},
+                         std::integral_constant<int, k % 2>{}, step + k);
+        });
     }
 
     // D[token, feature]: lane holds feature l32, tokens 8 * (v / 4) + 4 * kh + v % 4
@@ -395,11 +391,11 @@ int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, h
     } else if (tile.bt == 256) {
         st = launch_tiled<2, 4, 4, 2, 32>(x, w, bias, y, T, M, N, s);
     } else if (tile.bf == 256) {
-        st = launch_tiled<2, 4, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+        st = launch_tiled<2, 4, 2, 2, 64, 4>(x, w, bias, y, T, M, N, s);
     } else if (tile.bf == 128) {
-        st = launch_tiled<2, 2, 2, 2, 64>(x, w, bias, y, T, M, N, s);
+        st = launch_tiled<2, 2, 2, 2, 64, 4>(x, w, bias, y, T, M, N, s);
     } else {
-        st = launch_tiled<2, 2, 1, 1, 128>(x, w, bias, y, T, M, N, s);
+        st = launch_tiled<2, 2, 1, 1, 128, 4>(x, w, bias, y, T, M, N, s);
     }
     if (st != BS_OK) return st;
     BS_LAUNCH_CHECK();
