@@ -603,6 +603,14 @@ static int wide_choice(int I, int M, int N, int K, int T) {
     const bool walked = wide_partials(I, M, N, K, T) > 0, panel = bs_panel_partials(I, M, N, K, T) > 0;
     if (mode == BS_PREFILL_WALKED) return walked ? 1 : 0;
     if (mode == BS_PREFILL_PANEL) return panel ? 2 : 0;
+    // Both take the shape: the walked kernel requests its sign words strip by strip (16 bytes per row and request, every
+    // line eight times from L2), which costs more the more blocks there are and the more rows share a column range; the
+    // panel kernel requests four strips at a time but pays two barriers and an LDS round trip of the weight tile per
+    // strip.  Measured on the four 8B shapes, 2 to 8 blocks, 49 to 96 tokens: the panel kernel is ahead from 6 blocks
+    // on the tall shapes (14336 x 4096: 78 against 80 us at 6 blocks, 91 against 101 at 8) and from 5 blocks above 80
+    // tokens (214 against 221 us over the four layers at 6 blocks, 244 against 266 at 8); the walked kernel elsewhere
+    // (by 10 to 25 % up to 4 blocks).
+    if (walked && panel) return ((I >= 6 && M > N) || (T > 80 && I >= 5)) ? 2 : 1;
     return walked ? 1 : panel ? 2 : 0;
 }
 

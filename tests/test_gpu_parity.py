@@ -322,10 +322,20 @@ WIDE_CASES = [(2, 128, 128, 49, 16), (3, 1000, 1152, 64, 16), (1, 4096, 4096, 96
               (4, 130, 2432, 81, 12), (6, 2000, 1024, 49, 1)]
 
 
+@pytest.fixture
+def prefill_kernel():
+    """Lets a test pin the kernel of a forward of 49 tokens or more; back to the planner's choice afterwards."""
+    L = _lib.lib()
+    yield lambda mode: _lib.check(L.bs_set_prefill_kernel(mode), "bs_set_prefill_kernel")
+    L.bs_set_prefill_kernel(_lib.PREFILL_AUTO)
+
+
 @pytest.mark.parametrize("I,M,N,T,K", WIDE_CASES)
-def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K):
+def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K, prefill_kernel):
     print(f"forward walked strips I={I} M={M} N={N} T={T} K={K}", flush=True)
     L = _lib.lib()
+    prefill_kernel(_lib.PREFILL_WALKED)          # (from six blocks on a tall shape the planner prefers the panel kernel)
+    assert L.bs_forward_path(I, M, N, K, T) == _lib.PATH_WALKED
     # the path is taken: the scratch is g x ([T, M] partial sums + T sums of squares) for g column groups, not the weight
     need = int(L.bs_workspace_bytes(I, M, N, K, T))
     groups = need // (T * (M + 1) * 4)
@@ -345,14 +355,6 @@ def test_forward_49_to_96_tokens_matches_oracle(I, M, N, T, K):
     w = IU.unpack_and_reconstruct_w_hip(qd, ud, vd)
     dense = IU.linear_f16_hip(xd, w, bd).cpu().numpy()
     assert_close(y, dense, "vs rebuilt weight x dense kernel", 2e-3, 2e-4)
-
-
-@pytest.fixture
-def prefill_kernel():
-    """Lets a test pin the kernel of a forward of 49 tokens or more; back to the planner's choice afterwards."""
-    L = _lib.lib()
-    yield lambda mode: _lib.check(L.bs_set_prefill_kernel(mode), "bs_set_prefill_kernel")
-    L.bs_set_prefill_kernel(_lib.PREFILL_AUTO)
 
 
 # up to 128 tokens: sign tiles decoded into LDS and multiplied at once (128 rows x 128 tokens per workgroup): ragged
@@ -421,6 +423,9 @@ def test_planner_picks_walked_strips_then_panel_then_rebuild(prefill_kernel):
     assert path(3, 8192, 4096, 64) == _lib.PATH_WALKED        # 512 workgroups: the walked kernel fills the chip
     assert path(8, 4096, 14336, 64) == _lib.PATH_WALKED
     assert path(8, 14336, 4096, 64) == _lib.PATH_PANEL        # 448 workgroups for 512 slots: the walked kernel declines
+    assert path(8, 8192, 4096, 64) == _lib.PATH_PANEL         # both take it: six blocks and more on a tall shape go to the panel kernel
+    assert path(5, 8192, 4096, 64) == _lib.PATH_WALKED
+    assert path(5, 4096, 4096, 96) == _lib.PATH_PANEL and path(4, 4096, 4096, 96) == _lib.PATH_WALKED   # above 80 tokens from five blocks
     assert path(3, 14336, 4096, 64) == _lib.PATH_PANEL
     assert path(20, 4096, 4096, 64) == _lib.PATH_REBUILD      # vt of 20 blocks: no room for two walked workgroups, too many for the panel
     assert path(8, 4096, 4096, 97) == _lib.PATH_PANEL         # seven token tiles: beyond the walked kernel
