@@ -369,7 +369,7 @@ static LinearTile linear_tile(int T, int M, int N, bool aligned) {
     const auto wgs = [&](int bt, int bf) { return bs_cdiv(T, bt) * bs_cdiv(M, bf); };
     return wgs(256, 256) >= 160 ? LinearTile{256, 256, N % 64 == 0 ? 64 : 32} :
            wgs(128, 256) >= 160 ? LinearTile{128, 256, 64} :
-           wgs(128, 128) >= 192 ? LinearTile{128, 128, 64} : LinearTile{64, 64, 128};
+           wgs(128, 128) >= 160 ? LinearTile{128, 128, 64} : LinearTile{64, 64, 128};
 }
 
 int bs_launch_linear_f16(const half_t *x, const half_t *w, const half_t *bias, half_t *y,
