@@ -95,6 +95,21 @@ def test_dense_large_tiles_match_fp32_and_the_small_tile(T, M, N, tile, ktail):
         assert float((part != small).float().mean()) < 0.05                   # all but a few last-bit ties agree
 
 
+def test_dense_rows_too_long_for_32_bit_tile_offsets_take_the_generic_kernel():
+    """The tiled kernels address a tile's rows by 32-bit byte offsets from its origin (256 rows x N x 2 bytes must stay
+    below 4 GiB): from 2^23 columns the one-output-per-wave kernel runs instead, with the same result."""
+    T, M, N = 2, 3, (1 << 23) + 64
+    assert _lib.linear_plan(T, M, N)[:2] == (0, 0) and _lib.linear_plan(T, M, (1 << 23) - 64)[:2] != (0, 0)
+    g = torch.Generator(device=dev()).manual_seed(5)
+    x = (torch.randn(T, N, device=dev(), generator=g) * 0.05).half()
+    w = (torch.randn(M, N, device=dev(), generator=g) * 0.05).half()
+    y = IU.linear_f16_hip(x, w, None)
+    want = x.double() @ w.double().T
+    mx, mn = rel(y, want)
+    print(f"dense N={N}: max_rel={mx:.3e} mean_rel={mn:.3e}", flush=True)
+    assert mx <= 2e-3 and mn <= 1e-3
+
+
 def spot_rows_exact(q, u, vt, x, rows, bias=None):
     M, N = u.shape[1], vt.shape[2]
     qs = np.stack([qq.cpu().numpy().reshape(M, N // 8)[rows].reshape(-1) for qq in q])
